@@ -1,0 +1,55 @@
+"""Builds fbcunn_amd/libfbfftconv.so (HIP kernels + C ABI) for gfx950 with hipcc.
+
+    python -m fbcunn_amd.build            # compile and link
+    python -m fbcunn_amd.build --report   # also print register/LDS use per kernel
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "libfbfftconv.so")
+SOURCES = ["api.cpp", "fft_kernels.hip", "cgemm_kernels.hip", "bias_kernels.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
+    # packed fp32 VALU forms are switched off for every device function
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+]
+
+
+def _compile(src, report):
+    out = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", out]
+    if report:
+        cmd.append("-Rpass-analysis=kernel-resource-usage")
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on %s:\n%s" % (src, r.stderr))
+    return out, r.stderr
+
+
+def build(report=False):
+    os.makedirs(OBJ, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        results = list(ex.map(lambda s: _compile(s, report), SOURCES))
+    objs = [o for o, _ in results]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s" % r.stderr)
+    if report:
+        for _, err in results:
+            keep = [l for l in err.splitlines()
+                    if any(k in l for k in ("Function Name", "VGPRs:", "AGPRs", "ScratchSize", "Occupancy",
+                                            "LDS Size", "SGPRs:"))]
+            print("\n".join(keep))
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(report="--report" in sys.argv))

@@ -1,0 +1,412 @@
+// C ABI of the FFT-convolution library: argument checking, FFT-size planning,
+// frequency-buffer ownership and the stage schedule of the three passes.
+// Everything the reference spreads over fbcunn/SpatialConvolutionFFT.lua
+// (planning, buffers), fbcunn/SpatialConvolutionFBFFT.lua (the three passes) and
+// the FFI/luaT bindings (src/fft/FFTWrapperLua.cpp, src/MM.cu,
+// src/ConvolutionBias.cu) sits behind these entry points.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "../../include/fbfftconv.h"
+#include "kernels.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string &msg)
+{
+    g_last_error = msg;
+    return code;
+}
+
+int fail_hip(hipError_t e, const char *what)
+{
+    return fail(FBFC_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+constexpr int kMinFft = 8;
+constexpr int kMaxFft = 64;
+
+// fbcunn/SpatialConvolutionFFT.lua:875-882 (2^i, i = 1..10)
+int next_power_of_2(int v)
+{
+    for (int i = 1; i <= 10; ++i)
+        if ((1 << i) >= v) return 1 << i;
+    return -1;
+}
+
+int imax(int a, int b) { return a > b ? a : b; }
+
+int plan_query(const fbfc_conv_desc *d, fbfc_plan_info *info)
+{
+    if (d == nullptr || info == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (d->batch < 1 || d->in_planes < 1 || d->out_planes < 1 || d->in_h < 1 || d->in_w < 1 ||
+        d->k_h < 1 || d->k_w < 1)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    if (d->stride_h != 1 || d->stride_w != 1)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "fft only supports stride-1 convolutions atm");
+    if (d->pad_h < 0 || d->pad_w < 0)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "padding must be non-negative");
+    if (d->pad_h >= d->k_h || d->pad_w >= d->k_w)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "Padding must be smaller than kernel");
+    const int out_h = d->in_h + 2 * d->pad_h - d->k_h + 1;
+    const int out_w = d->in_w + 2 * d->pad_w - d->k_w + 1;
+    if (out_h < 1 || out_w < 1)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "kernel larger than padded input");
+    // prepareFBFFTSizeAndBuffers: square, power of two, covers every operand
+    int need = imax(imax(d->in_h + 2 * d->pad_h, d->in_w + 2 * d->pad_w), imax(d->k_h, d->k_w));
+    need = imax(need, imax(out_h, out_w));
+    int n = next_power_of_2(need);
+    if (n < 0) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "Too large a convolution dimensions");
+    if (n < kMinFft) n = kMinFft;  // a larger canvas gives the same convolution
+    if (n > kMaxFft) {
+        char buf[96];
+        std::snprintf(buf, sizeof buf, "FFT size %d not supported (8..%d)", n, kMaxFft);
+        return fail(FBFC_ERR_UNSUPPORTED_SIZE, buf);
+    }
+    const size_t q = (size_t)n * (n / 2 + 1);
+    info->fft_size = n;
+    info->n_freq = (int)q;
+    info->out_h = out_h;
+    info->out_w = out_w;
+    info->input_freq_bytes = q * d->batch * d->in_planes * 8;
+    info->weight_freq_bytes = q * d->out_planes * d->in_planes * 8;
+    info->output_freq_bytes = q * d->batch * d->out_planes * 8;
+    info->scratch_bytes = fbfc::bias_grad_scratch_bytes(d->batch, d->out_planes);
+    return FBFC_OK;
+}
+
+bool fft_size_ok(int n) { return n == 8 || n == 16 || n == 32 || n == 64; }
+
+}  // namespace
+
+struct fbfc_plan {
+    fbfc_conv_desc d;
+    fbfc_plan_info info;
+    int device;
+    float *in_freq, *w_freq, *out_freq, *res_freq, *scratch;
+    unsigned reuse;
+    bool have_in, have_w, have_out;  // which forward spectra are valid in their buffer
+    int timed;
+    hipEvent_t ev[FBFC_NUM_STAGES + 1];
+    bool ev_made;
+    float stage_ms[FBFC_NUM_STAGES];
+};
+
+namespace {
+
+// Records stage boundaries when the plan is timed.
+struct StageTimer {
+    fbfc_plan *p;
+    hipStream_t s;
+    int n;
+    int slot[FBFC_NUM_STAGES];
+    StageTimer(fbfc_plan *plan, hipStream_t stream) : p(plan), s(stream), n(0)
+    {
+        if (p->timed) {
+            for (float &m : p->stage_ms) m = 0.0f;
+            (void)hipEventRecord(p->ev[0], s);
+        }
+    }
+    void done(int stage)
+    {
+        if (!p->timed) return;
+        slot[n] = stage;
+        ++n;
+        (void)hipEventRecord(p->ev[n], s);
+    }
+    int finish()
+    {
+        if (!p->timed) return FBFC_OK;
+        hipError_t e = hipEventSynchronize(p->ev[n]);
+        if (e != hipSuccess) return fail_hip(e, "hipEventSynchronize");
+        for (int i = 0; i < n; ++i) {
+            float ms = 0.0f;
+            e = hipEventElapsedTime(&ms, p->ev[i], p->ev[i + 1]);
+            if (e != hipSuccess) return fail_hip(e, "hipEventElapsedTime");
+            p->stage_ms[slot[i]] = ms;
+        }
+        return FBFC_OK;
+    }
+};
+
+#define FBFC_TRY(expr, what)                                   \
+    do {                                                       \
+        hipError_t e_ = (expr);                                \
+        if (e_ != hipSuccess) return fail_hip(e_, what);       \
+    } while (0)
+
+}  // namespace
+
+extern "C" {
+
+const char *fbfc_version(void) { return "fbfftconv 0.1 (gfx950)"; }
+
+const char *fbfc_last_error(void) { return g_last_error.c_str(); }
+
+int fbfc_plan_query(const fbfc_conv_desc *desc, fbfc_plan_info *info)
+{
+    return plan_query(desc, info);
+}
+
+int fbfc_plan_create(const fbfc_conv_desc *desc, fbfc_plan **out)
+{
+    if (out == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    *out = nullptr;
+    fbfc_plan_info info;
+    const int rc = plan_query(desc, &info);
+    if (rc != FBFC_OK) return rc;
+    fbfc_plan *p = new (std::nothrow) fbfc_plan();
+    if (p == nullptr) return fail(FBFC_ERR_OUT_OF_MEMORY, "host allocation failed");
+    std::memset(p, 0, sizeof *p);
+    p->d = *desc;
+    p->info = info;
+    hipError_t e = hipGetDevice(&p->device);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->in_freq), info.input_freq_bytes);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->w_freq), info.weight_freq_bytes);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->out_freq), info.output_freq_bytes);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->scratch), info.scratch_bytes);
+    if (e != hipSuccess) {
+        const bool oom = (e == hipErrorOutOfMemory);
+        (void)hipGetLastError();
+        fbfc_plan_destroy(p);
+        // the reference reports "Not enough memory for FFT buffers" (SpatialConvolutionFFT.lua:687)
+        if (oom) return fail(FBFC_ERR_OUT_OF_MEMORY, "Not enough memory for FFT buffers");
+        return fail_hip(e, "plan allocation");
+    }
+    *out = p;
+    return FBFC_OK;
+}
+
+int fbfc_plan_destroy(fbfc_plan *p)
+{
+    if (p == nullptr) return FBFC_OK;
+    if (p->in_freq) (void)hipFree(p->in_freq);
+    if (p->w_freq) (void)hipFree(p->w_freq);
+    if (p->out_freq) (void)hipFree(p->out_freq);
+    if (p->res_freq) (void)hipFree(p->res_freq);
+    if (p->scratch) (void)hipFree(p->scratch);
+    if (p->ev_made)
+        for (hipEvent_t &ev : p->ev) (void)hipEventDestroy(ev);
+    delete p;
+    return FBFC_OK;
+}
+
+int fbfc_plan_get_info(const fbfc_plan *p, fbfc_plan_info *info)
+{
+    if (p == nullptr || info == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    *info = p->info;
+    return FBFC_OK;
+}
+
+int fbfc_plan_set_reuse(fbfc_plan *p, unsigned flags)
+{
+    if (p == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null plan");
+    if (flags & ~(unsigned)FBFC_REUSE_ALL) return fail(FBFC_ERR_INVALID_ARGUMENT, "unknown memory reuse policy");
+    if (flags != 0 && p->res_freq == nullptr) {
+        // With reuse, a pass must not overwrite a spectrum a later pass wants: its
+        // result goes to a buffer of its own (the reference keys such buffers by
+        // "isOutputOfAlgorithm", SpatialConvolutionFBFFT.lua:382-399).
+        size_t bytes = p->info.input_freq_bytes;
+        if (p->info.weight_freq_bytes > bytes) bytes = p->info.weight_freq_bytes;
+        if (p->info.output_freq_bytes > bytes) bytes = p->info.output_freq_bytes;
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&p->res_freq), bytes);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(FBFC_ERR_OUT_OF_MEMORY, "Not enough memory for FFT buffers");
+        }
+    }
+    p->reuse = flags;
+    p->have_in = p->have_w = p->have_out = false;
+    return FBFC_OK;
+}
+
+int fbfc_plan_set_timed(fbfc_plan *p, int on)
+{
+    if (p == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null plan");
+    if (on && !p->ev_made) {
+        for (hipEvent_t &ev : p->ev) FBFC_TRY(hipEventCreate(&ev), "hipEventCreate");
+        p->ev_made = true;
+    }
+    p->timed = on ? 1 : 0;
+    return FBFC_OK;
+}
+
+int fbfc_plan_stage_ms(const fbfc_plan *p, float *ms, int n)
+{
+    if (p == nullptr || ms == nullptr || n < 0) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    for (int i = 0; i < n; ++i) ms[i] = (i < FBFC_NUM_STAGES) ? p->stage_ms[i] : 0.0f;
+    return FBFC_OK;
+}
+
+int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, const float *bias,
+                       float *output, void *stream)
+{
+    if (p == nullptr || input == nullptr || weight == nullptr || output == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const fbfc_conv_desc &d = p->d;
+    const int N = p->info.fft_size, Q = p->info.n_freq;
+    StageTimer tm(p, s);
+    FBFC_TRY(fbfc::launch_rfft2d(N, input, p->in_freq, (long)d.batch * d.in_planes, d.in_h, d.in_w,
+                                 d.pad_h, d.pad_w, s), "rfft2d(input)");
+    p->have_in = true;
+    tm.done(FBFC_STAGE_FFT_A);
+    FBFC_TRY(fbfc::launch_rfft2d(N, weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w,
+                                 0, 0, s), "rfft2d(weight)");
+    p->have_w = true;
+    tm.done(FBFC_STAGE_FFT_B);
+    float *res = p->reuse ? p->res_freq : p->out_freq;
+    if (!p->reuse) p->have_out = false;
+    // O[b][f] = 1/N^2 sum_p I[b][p] conj(W[f][p])   (SpatialConvolutionFBFFT.lua:157-164)
+    FBFC_TRY(fbfc::launch_cgemm_freq(0, p->in_freq, p->w_freq, res, Q, d.batch, d.out_planes,
+                                     d.in_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(fprop)");
+    tm.done(FBFC_STAGE_MM);
+    FBFC_TRY(fbfc::launch_irfft2d(N, res, output, (long)d.batch * d.out_planes, p->info.out_h,
+                                  p->info.out_w, 0, 0, bias, d.out_planes, s), "irfft2d(output)");
+    tm.done(FBFC_STAGE_IFFT);
+    return tm.finish();
+}
+
+int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *weight,
+                           float *grad_input, void *stream)
+{
+    if (p == nullptr || grad_output == nullptr || weight == nullptr || grad_input == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const fbfc_conv_desc &d = p->d;
+    const int N = p->info.fft_size, Q = p->info.n_freq;
+    StageTimer tm(p, s);
+    FBFC_TRY(fbfc::launch_rfft2d(N, grad_output, p->out_freq, (long)d.batch * d.out_planes,
+                                 p->info.out_h, p->info.out_w, 0, 0, s), "rfft2d(gradOutput)");
+    p->have_out = true;
+    tm.done(FBFC_STAGE_FFT_A);
+    if (!((p->reuse & FBFC_REUSE_WEIGHT) && p->have_w)) {
+        FBFC_TRY(fbfc::launch_rfft2d(N, weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h,
+                                     d.k_w, 0, 0, s), "rfft2d(weight)");
+        p->have_w = true;
+        tm.done(FBFC_STAGE_FFT_B);
+    }
+    float *res = p->reuse ? p->res_freq : p->in_freq;
+    if (!p->reuse) p->have_in = false;
+    // GI[b][p] = 1/N^2 sum_f GO[b][f] W[f][p]   (SpatialConvolutionFBFFT.lua:244-251)
+    FBFC_TRY(fbfc::launch_cgemm_freq(1, p->out_freq, p->w_freq, res, Q, d.batch, d.in_planes,
+                                     d.out_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(bprop)");
+    tm.done(FBFC_STAGE_MM);
+    FBFC_TRY(fbfc::launch_irfft2d(N, res, grad_input, (long)d.batch * d.in_planes, d.in_h, d.in_w,
+                                  d.pad_h, d.pad_w, nullptr, 1, s), "irfft2d(gradInput)");
+    tm.done(FBFC_STAGE_IFFT);
+    return tm.finish();
+}
+
+int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad_output,
+                             float *grad_weight, float *grad_bias, float scale, void *stream)
+{
+    if (p == nullptr || input == nullptr || grad_output == nullptr || grad_weight == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const fbfc_conv_desc &d = p->d;
+    const int N = p->info.fft_size, Q = p->info.n_freq;
+    StageTimer tm(p, s);
+    if (grad_bias != nullptr) {
+        FBFC_TRY(fbfc::launch_bias_grad(grad_output, grad_bias, scale, d.batch, d.out_planes,
+                                        p->info.out_h * p->info.out_w, p->scratch, s), "bias grad");
+        tm.done(FBFC_STAGE_BIAS_GRAD);
+    }
+    if (!((p->reuse & FBFC_REUSE_OUTPUT) && p->have_out)) {
+        FBFC_TRY(fbfc::launch_rfft2d(N, grad_output, p->out_freq, (long)d.batch * d.out_planes,
+                                     p->info.out_h, p->info.out_w, 0, 0, s), "rfft2d(gradOutput)");
+        p->have_out = true;
+        tm.done(FBFC_STAGE_FFT_A);
+    }
+    if (!((p->reuse & FBFC_REUSE_INPUT) && p->have_in)) {
+        FBFC_TRY(fbfc::launch_rfft2d(N, input, p->in_freq, (long)d.batch * d.in_planes, d.in_h,
+                                     d.in_w, d.pad_h, d.pad_w, s), "rfft2d(input)");
+        p->have_in = true;
+        tm.done(FBFC_STAGE_FFT_B);
+    }
+    float *res = p->reuse ? p->res_freq : p->w_freq;
+    if (!p->reuse) p->have_w = false;
+    // GW[f][p] = scale/N^2 sum_b conj(GO[b][f]) I[b][p]   (SpatialConvolutionFBFFT.lua:337-344)
+    FBFC_TRY(fbfc::launch_cgemm_freq(2, p->out_freq, p->in_freq, res, Q, d.out_planes, d.in_planes,
+                                     d.batch, scale / ((float)N * (float)N), 0, s), "cgemm(accGrad)");
+    tm.done(FBFC_STAGE_MM);
+    FBFC_TRY(fbfc::launch_irfft2d(N, res, grad_weight, (long)d.out_planes * d.in_planes, d.k_h, d.k_w,
+                                  0, 0, nullptr, 1, s), "irfft2d(gradWeight)");
+    tm.done(FBFC_STAGE_IFFT);
+    return tm.finish();
+}
+
+int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
+               float *freq, void *stream)
+{
+    if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!fft_size_ok(fft_size)) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
+    if (planes < 1 || h < 1 || w < 1 || pad_u < 0 || pad_l < 0 || h + pad_u > fft_size ||
+        w + pad_l > fft_size)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "plane plus padding must fit the FFT size");
+    FBFC_TRY(fbfc::launch_rfft2d(fft_size, real, freq, planes, h, w, pad_u, pad_l,
+                                 static_cast<hipStream_t>(stream)), "rfft2d");
+    return FBFC_OK;
+}
+
+int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
+                float *real, const float *bias, int bias_period, void *stream)
+{
+    if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!fft_size_ok(fft_size)) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
+    if (planes < 1 || h < 1 || w < 1 || pad_u < 0 || pad_l < 0 || h + pad_u > fft_size ||
+        w + pad_l > fft_size)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "plane plus padding must fit the FFT size");
+    if (bias != nullptr && bias_period < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "bias_period must be positive");
+    FBFC_TRY(fbfc::launch_irfft2d(fft_size, freq, real, planes, h, w, pad_u, pad_l, bias, bias_period,
+                                  static_cast<hipStream_t>(stream)), "irfft2d");
+    return FBFC_OK;
+}
+
+int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq, int m, int n, int k,
+                      float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate, void *stream)
+{
+    if (A == nullptr || B == nullptr || C == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (n_freq < 1 || m < 1 || n < 1 || k < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    if (conj_trans_a && conj_trans_b)
+        return fail(FBFC_ERR_UNSUPPORTED_DIMENSION, "conjugate-transposing both operands is not supported");
+    const int mode = conj_trans_b ? 0 : (conj_trans_a ? 2 : 1);
+    FBFC_TRY(fbfc::launch_cgemm_freq(mode, A, B, C, n_freq, m, n, k, inv_norm, accumulate ? 1 : 0,
+                                     static_cast<hipStream_t>(stream)), "cgemm");
+    return FBFC_OK;
+}
+
+int fbfc_update_output_bias(float *output, const float *bias, int batch, int planes, int h, int w,
+                            void *stream)
+{
+    if (output == nullptr || bias == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (batch < 1 || planes < 1 || h < 1 || w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    FBFC_TRY(fbfc::launch_bias_add(output, bias, batch, planes, h * w, static_cast<hipStream_t>(stream)),
+             "bias add");
+    return FBFC_OK;
+}
+
+size_t fbfc_bias_grad_scratch_bytes(int batch, int planes)
+{
+    if (batch < 1 || planes < 1) return 0;
+    return fbfc::bias_grad_scratch_bytes(batch, planes);
+}
+
+int fbfc_acc_grad_parameters_bias(const float *grad_output, float *grad_bias, float scale, int batch,
+                                  int planes, int h, int w, float *scratch, void *stream)
+{
+    if (grad_output == nullptr || grad_bias == nullptr || scratch == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (batch < 1 || planes < 1 || h < 1 || w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    FBFC_TRY(fbfc::launch_bias_grad(grad_output, grad_bias, scale, batch, planes, h * w, scratch,
+                                    static_cast<hipStream_t>(stream)), "bias grad");
+    return FBFC_OK;
+}
+
+}  // extern "C"

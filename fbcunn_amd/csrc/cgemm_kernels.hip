@@ -1,0 +1,229 @@
+// Per-frequency complex contraction over planes as an fp32 MFMA GEMM (gfx950).
+//
+// Replaces transposeMMFFI -> fbcuda transposeMM (src/MM.cu:14-73) and the
+// cublasCgeam + cublasCgemmBatched pair of the Gemm module
+// (src/CuBLASWrapper.cpp:113-125, 437-452).  The three call sites
+// (fbcunn/SpatialConvolutionFBFFT.lua:157-164, 244-251, 337-344) map to modes
+// 0, 1, 2 below.  Operands are frequency-major, so each frequency is a dense
+// row-major complex matrix and no transpose kernel exists.
+//
+// A complex product is carried as a real GEMM with doubled inner dimension:
+//   C_re = sum_k' A'[m][k'] Bre'[k'][n],  C_im = sum_k' A'[m][k'] Bim'[k'][n]
+// where k' enumerates (k, re|im).  A' is the interleaved storage read as it
+// lies; Bre'/Bim' are B with its components swapped and sign-flipped in
+// registers.  v_mfma_f32_32x32x2_f32 takes the two k' of a step from the two
+// half-waves; because a sum may run over k' in any order, each half-wave is
+// given the k' that are contiguous for it in LDS.
+//
+// Workgroup: 256 lanes = 4 waves in 2x2, each wave a 32x32 complex block
+// (2 x 16 accumulator registers); tile 64 x 64 x 16 complex per step with
+// register-prefetch double buffering through LDS.
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace fbfc {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 64, BN = 64, KT = 16;
+constexpr int LDK = 2 * KT + 4;  // floats per row of a K-contiguous tile [64][KT] (+16 B pad)
+constexpr int LDM = 2 * 64;      // floats per row of a row-contiguous tile [KT][64]
+constexpr int TILE_FLOATS_KC = 64 * LDK;
+constexpr int TILE_FLOATS_MC = KT * LDM;
+constexpr int TILE_FLOATS = TILE_FLOATS_KC > TILE_FLOATS_MC ? TILE_FLOATS_KC : TILE_FLOATS_MC;
+
+// Loads one operand tile (1024 complex = 4 per lane) into registers.
+//   KC == true : matrix is [rows][K], tile covers rows r0.. (64) x k0.. (KT)
+//   KC == false: matrix is [K][cols], tile covers k0.. (KT) x c0.. (64)
+template <bool KC>
+__device__ __forceinline__ void load_tile(const float2 *__restrict__ M, int ld, int nrows_total,
+                                          int ncols_total, int r0, int c0, int tid, float2 (&v)[4])
+{
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = tid + 256 * i;
+        int r, c;
+        if (KC) { r = e / KT; c = e % KT; } else { r = e / 64; c = e % 64; }
+        const int gr = r0 + r, gc = c0 + c;
+        v[i] = (gr < nrows_total && gc < ncols_total) ? M[(long)gr * ld + gc] : make_float2(0.f, 0.f);
+    }
+}
+
+template <bool KC>
+__device__ __forceinline__ void store_tile(float *lds, int tid, const float2 (&v)[4])
+{
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = tid + 256 * i;
+        int r, c;
+        if (KC) { r = e / KT; c = e % KT; } else { r = e / 64; c = e % 64; }
+        float2 *p = reinterpret_cast<float2 *>(lds + r * (KC ? LDK : LDM) + 2 * c);
+        *p = v[i];
+    }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restrict__ A,
+                                                         const float2 *__restrict__ B,
+                                                         float2 *__restrict__ C, int M, int N, int K,
+                                                         float alpha, int accumulate, int tilesM,
+                                                         int tilesN, int total_wgs, int chunk)
+{
+    constexpr bool A_KC = (MODE != 2);
+    constexpr bool B_KC = (MODE == 0);
+    __shared__ __align__(16) float As[2][TILE_FLOATS];
+    __shared__ __align__(16) float Bs[2][TILE_FLOATS];
+
+    // Workgroups are handed to the 8 XCDs round-robin; remap so that each XCD
+    // works on a contiguous range of (frequency, tile) and the tiles of one
+    // frequency share that XCD's L2.
+    const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
+    if (wg >= total_wgs) return;
+    const int tiles = tilesM * tilesN;
+    const int q = wg / tiles;
+    const int tile = wg - q * tiles;
+    const int m0 = (tile / tilesN) * BM;
+    const int n0 = (tile % tilesN) * BN;
+
+    const float2 *Aq = A + (long)q * M * K;
+    const float2 *Bq = B + (long)q * N * K;
+    float2 *Cq = C + (long)q * M * N;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, h = lane >> 5;
+
+    floatx16 cre, cim;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { cre[r] = 0.f; cim[r] = 0.f; }
+
+    float2 pa[4], pb[4];
+    const int nk = (K + KT - 1) / KT;
+
+    auto gload = [&](int kt) {
+        const int k0 = kt * KT;
+        if (A_KC) load_tile<true>(Aq, K, M, K, m0, k0, tid, pa);   // A[m][k]
+        else      load_tile<false>(Aq, M, K, M, k0, m0, tid, pa);  // A[k][m]
+        if (B_KC) load_tile<true>(Bq, K, N, K, n0, k0, tid, pb);   // B[n][k]
+        else      load_tile<false>(Bq, N, K, N, k0, n0, tid, pb);  // B[k][n]
+    };
+    auto sstore = [&](int buf) {
+        store_tile<A_KC>(As[buf], tid, pa);
+        store_tile<B_KC>(Bs[buf], tid, pb);
+    };
+
+    gload(0);
+    sstore(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) gload(kt + 1);
+
+        const float *as = As[buf];
+        const float *bs = Bs[buf];
+        const int arow = 32 * wm + li;  // row of the A' operand this lane feeds
+        const int bcol = 32 * wn + li;  // column of the B' operand this lane feeds
+
+        if (MODE == 0) {
+            // both K-contiguous: half-wave h owns complex k in [8h, 8h+8) = 16 consecutive floats
+            float a[16], b[16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 va = *reinterpret_cast<const float4 *>(as + arow * LDK + 16 * h + 4 * j);
+                const float4 vb = *reinterpret_cast<const float4 *>(bs + bcol * LDK + 16 * h + 4 * j);
+                a[4 * j] = va.x; a[4 * j + 1] = va.y; a[4 * j + 2] = va.z; a[4 * j + 3] = va.w;
+                b[4 * j] = vb.x; b[4 * j + 1] = vb.y; b[4 * j + 2] = vb.z; b[4 * j + 3] = vb.w;
+            }
+#pragma unroll
+            for (int s = 0; s < 16; s += 2) {
+                // k' = (k, re): A' = a_re ; k' = (k, im): A' = a_im.   C = A conj(B)
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], -b[s + 1], cim, 0, 0, 0);
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s + 1], b[s + 1], cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s + 1], b[s], cim, 0, 0, 0);
+            }
+        } else if (MODE == 1) {
+            // A K-contiguous (as above); B row-contiguous [k][n]: one (re,im) pair per two steps
+            float a[16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 va = *reinterpret_cast<const float4 *>(as + arow * LDK + 16 * h + 4 * j);
+                a[4 * j] = va.x; a[4 * j + 1] = va.y; a[4 * j + 2] = va.z; a[4 * j + 3] = va.w;
+            }
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDM + 2 * bcol);
+                // C = A B
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.x, cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.y, cim, 0, 0, 0);
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], -vb.y, cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], vb.x, cim, 0, 0, 0);
+            }
+        } else {
+            // both row-contiguous [k][.]: step s is complex k = s; half-wave 0 feeds the real
+            // part of A, half-wave 1 the imaginary part.   C = conj(A)^T B
+#pragma unroll
+            for (int s = 0; s < KT; ++s) {
+                const float av = as[s * LDM + 2 * arow + h];
+                const float2 vb = *reinterpret_cast<const float2 *>(bs + s * LDM + 2 * bcol);
+                const float opre = h ? vb.y : vb.x;
+                const float opim = h ? -vb.x : vb.y;
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(av, opre, cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(av, opim, cim, 0, 0, 0);
+            }
+        }
+
+        if (kt + 1 < nk) {
+            sstore(buf ^ 1);  // the other buffer was last read before the previous barrier
+            __syncthreads();
+        }
+    }
+
+    // epilogue: accumulator register r of lane (li, h) is C[8*(r/4) + 4*h + r%4][li] of the block
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int row = m0 + 32 * wm + 8 * (r / 4) + 4 * h + (r % 4);
+        const int col = n0 + 32 * wn + li;
+        if (row < M && col < N) {
+            float2 v = make_float2(alpha * cre[r], alpha * cim[r]);
+            float2 *dst = Cq + (long)row * N + col;
+            if (accumulate) {
+                const float2 o = *dst;
+                v.x += o.x;
+                v.y += o.y;
+            }
+            *dst = v;
+        }
+    }
+}
+
+template <int MODE>
+static hipError_t launch_mode(const float *A, const float *B, float *C, int n_freq, int m, int n,
+                              int k, float alpha, int accumulate, hipStream_t s)
+{
+    const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
+    const long total = (long)n_freq * tilesM * tilesN;
+    if (total <= 0 || total > 0x7fffff00L) return hipErrorInvalidValue;
+    const int chunk = (int)((total + 7) / 8);
+    hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
+                       reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
+                       reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
+                       (int)total, chunk);
+    return hipGetLastError();
+}
+
+hipError_t launch_cgemm_freq(int mode, const float *A, const float *B, float *C, int n_freq, int m,
+                             int n, int k, float alpha, int accumulate, hipStream_t s)
+{
+    switch (mode) {
+        case 0: return launch_mode<0>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
+        case 1: return launch_mode<1>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
+        case 2: return launch_mode<2>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace fbfc

@@ -1,0 +1,30 @@
+// Internal launch interface between the C ABI (api.cpp) and the kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+namespace fbfc {
+
+// fft_kernels.hip ------------------------------------------------------------
+// N in {8,16,32,64}; any other value returns hipErrorInvalidValue.
+hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
+                         int padL, hipStream_t s);
+hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
+                          int padL, const float *bias, int bias_period, hipStream_t s);
+
+// cgemm_kernels.hip ------------------------------------------------------------
+// mode 0: C[m][n] (+)= alpha * sum_k A[m][k] * conj(B[n][k])   A (m x k), B (n x k)
+// mode 1: C[m][n] (+)= alpha * sum_k A[m][k] * B[k][n]         A (m x k), B (k x n)
+// mode 2: C[m][n] (+)= alpha * sum_k conj(A[k][m]) * B[k][n]   A (k x m), B (k x n)
+// for each of n_freq frequencies; operands frequency-major, complex interleaved.
+hipError_t launch_cgemm_freq(int mode, const float *A, const float *B, float *C, int n_freq, int m,
+                             int n, int k, float alpha, int accumulate, hipStream_t s);
+
+// bias_kernels.hip ---------------------------------------------------------------
+hipError_t launch_bias_add(float *out, const float *bias, int batch, int planes, int hw,
+                           hipStream_t s);
+size_t bias_grad_scratch_bytes(int batch, int planes);
+hipError_t launch_bias_grad(const float *grad_out, float *grad_bias, float scale, int batch,
+                            int planes, int hw, float *scratch, hipStream_t s);
+
+}  // namespace fbfc

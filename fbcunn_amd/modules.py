@@ -1,0 +1,292 @@
+"""Host-side mirror of the reference's Lua modules for the FFT-convolution path.
+
+Same names, constructor arguments, fields and call protocol as
+nn.SpatialConvolutionFBFFT / nn.SpatialConvolutionFBFFTGemm
+(fbcunn/SpatialConvolutionFBFFT.lua, fbcunn/SpatialConvolutionFBFFTGemm.lua,
+base class fbcunn/SpatialConvolutionFFT.lua) and nn.FFTWrapper
+(fbcunn/FFTWrapper.lua).  All arithmetic happens in libfbfftconv.so; torch is
+used only to own device memory and to name the current stream.
+"""
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+from ._lib import ConvDesc, FbfcError, PlanInfo, check, lib
+
+__all__ = ["SpatialConvolutionFFT", "SpatialConvolutionFBFFT", "SpatialConvolutionFBFFTGemm",
+           "FFTWrapper", "transposeMM", "updateOutputBias", "accGradParametersBias", "FbfcError"]
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check_tensor(t, name, ndim=None):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError("%s: CUDA support only!" % name)   # the reference's assert message
+    if t.dtype != torch.float32:
+        raise TypeError("%s must be float32" % name)
+    if ndim is not None and t.dim() != ndim:
+        raise ValueError("%s must be %d-D" % (name, ndim))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+
+
+class _Plan:
+    """RAII holder of one fbfc_plan."""
+
+    def __init__(self, desc):
+        self.handle = ctypes.c_void_p(0)
+        check(lib().fbfc_plan_create(ctypes.byref(desc), ctypes.byref(self.handle)))
+        self.info = PlanInfo()
+        check(lib().fbfc_plan_get_info(self.handle, ctypes.byref(self.info)))
+
+    def close(self):
+        if self.handle:
+            lib().fbfc_plan_destroy(self.handle)
+            self.handle = ctypes.c_void_p(0)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class SpatialConvolutionFFT:
+    """Module state and protocol of nn.SpatialConvolutionFFT
+    (fbcunn/SpatialConvolutionFFT.lua:150-316, 405-416)."""
+
+    memoryReuseNone = "none"
+    memoryReuseInput = "input"
+    memoryReuseOutput = "output"
+    memoryReuseWeight = "weight"
+    memoryReuseAll = "all"
+    _REUSE_BITS = {"none": _lib.REUSE_NONE, "input": _lib.REUSE_INPUT, "output": _lib.REUSE_OUTPUT,
+                   "weight": _lib.REUSE_WEIGHT, "all": _lib.REUSE_ALL}
+
+    def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padLeft=0, padUp=0,
+                 memoryReusePolicy=None, numCudaStreams=None, device="cuda"):
+        for v in (nInputPlane, nOutputPlane, kW, kH, dW, dH, padLeft, padUp):
+            if not isinstance(v, int):
+                raise TypeError("module dimensions must be numbers")
+        self.nInputPlane, self.nOutputPlane = nInputPlane, nOutputPlane
+        self.kW, self.kH = kW, kH
+        self.dW, self.dH = dW, dH
+        self.padLeft, self.padUp = padLeft, padUp
+        self.padRight, self.padDown = padLeft, padUp
+        if self.dW != 1 or self.dH != 1:
+            raise ValueError("fft only supports stride-1 convolutions atm")
+        if not (self.padUp < self.kH and self.padLeft < self.kW):
+            raise ValueError("Padding must be smaller than kernel")
+        if memoryReusePolicy is None:
+            memoryReusePolicy = [self.memoryReuseNone]
+        if isinstance(memoryReusePolicy, str):
+            memoryReusePolicy = [memoryReusePolicy]
+        self.memoryReusePolicy = list(memoryReusePolicy)
+        self._reuse_bits = 0
+        for p in self.memoryReusePolicy:
+            if p not in self._REUSE_BITS:
+                raise ValueError("unknown memory reuse policy " + str(p))
+            self._reuse_bits |= self._REUSE_BITS[p]
+        self.numCudaStreams = numCudaStreams or 16  # kept for signature parity; one stream is used
+        self.device = torch.device(device)
+        self.weight = torch.empty(nOutputPlane, nInputPlane, kH, kW, device=self.device)
+        self.bias = torch.empty(nOutputPlane, device=self.device)
+        self.gradWeight = torch.zeros(nOutputPlane, nInputPlane, kH, kW, device=self.device)
+        self.gradBias = torch.zeros(nOutputPlane, device=self.device)
+        self.output = None
+        self.gradInput = None
+        self.timed = False
+        self._plans = {}
+        self.reset()
+
+    # -- parameters ---------------------------------------------------------------
+    def reset(self, stdv=None):
+        """uniform(-stdv, stdv), stdv = 1/sqrt(kW*kH*nInputPlane) (SpatialConvolutionFFT.lua:271-289)."""
+        if stdv is not None:
+            stdv = stdv * math.sqrt(3)
+        else:
+            stdv = 1.0 / math.sqrt(self.kW * self.kH * self.nInputPlane)
+        self.weight.uniform_(-stdv, stdv)
+        self.bias.uniform_(-stdv, stdv)
+
+    def zeroGradParameters(self):
+        self.gradWeight.zero_()
+        self.gradBias.zero_()
+
+    def parameters(self):
+        return [self.weight, self.bias], [self.gradWeight, self.gradBias]
+
+    # -- planning -------------------------------------------------------------------
+    def _plan_for(self, batch, in_h, in_w):
+        key = (batch, in_h, in_w)
+        plan = self._plans.get(key)
+        if plan is None:
+            desc = ConvDesc(batch, self.nInputPlane, self.nOutputPlane, in_h, in_w, self.kH, self.kW,
+                            self.dH, self.dW, self.padUp, self.padLeft)
+            plan = _Plan(desc)
+            if self._reuse_bits:
+                check(lib().fbfc_plan_set_reuse(plan.handle, self._reuse_bits))
+            self._plans[key] = plan
+        check(lib().fbfc_plan_set_timed(plan.handle, 1 if self.timed else 0))
+        return plan
+
+    def _check_input(self, input):
+        _check_tensor(input, "input", 4)
+        if input.size(1) != self.nInputPlane:
+            raise ValueError("input has %d planes, module expects %d" % (input.size(1), self.nInputPlane))
+
+    def stageTimes(self, input):
+        """ms per stage of the last pass run with self.timed = True (dict)."""
+        plan = self._plan_for(input.size(0), input.size(2), input.size(3))
+        ms = (ctypes.c_float * len(_lib.STAGE_NAMES))()
+        check(lib().fbfc_plan_stage_ms(plan.handle, ms, len(_lib.STAGE_NAMES)))
+        return dict(zip(_lib.STAGE_NAMES, [float(x) for x in ms]))
+
+    # -- nn.Module protocol -----------------------------------------------------------
+    def updateOutput(self, input):
+        self._check_input(input)
+        B, _, H, W = input.shape
+        plan = self._plan_for(B, H, W)
+        shape = (B, self.nOutputPlane, plan.info.out_h, plan.info.out_w)
+        # allocated once, like the reference (SpatialConvolutionFFT.lua:435-441), but
+        # re-made when the shape changes instead of silently keeping the old size
+        if self.output is None or tuple(self.output.shape) != shape:
+            self.output = torch.empty(shape, device=input.device)
+        check(lib().fbfc_update_output(plan.handle, _ptr(input), _ptr(self.weight), _ptr(self.bias),
+                                       _ptr(self.output), _stream()))
+        return self.output
+
+    forward = updateOutput
+
+    def updateGradInput(self, input, gradOutput):
+        self._check_input(input)
+        _check_tensor(gradOutput, "gradOutput", 4)
+        B, _, H, W = input.shape
+        plan = self._plan_for(B, H, W)
+        if tuple(gradOutput.shape) != (B, self.nOutputPlane, plan.info.out_h, plan.info.out_w):
+            raise ValueError("gradOutput has the wrong shape")
+        if self.gradInput is None or self.gradInput.shape != input.shape:
+            self.gradInput = torch.empty_like(input)
+        check(lib().fbfc_update_grad_input(plan.handle, _ptr(gradOutput), _ptr(self.weight),
+                                           _ptr(self.gradInput), _stream()))
+        return self.gradInput
+
+    def accGradParameters(self, input, gradOutput, scale=1.0):
+        """gradWeight and gradBias are overwritten, as in the reference's FBFFT path
+        (accumulate=false, SpatialConvolutionFBFFT.lua:337-349)."""
+        self._check_input(input)
+        _check_tensor(gradOutput, "gradOutput", 4)
+        B, _, H, W = input.shape
+        plan = self._plan_for(B, H, W)
+        if tuple(gradOutput.shape) != (B, self.nOutputPlane, plan.info.out_h, plan.info.out_w):
+            raise ValueError("gradOutput has the wrong shape")
+        check(lib().fbfc_acc_grad_parameters(plan.handle, _ptr(input), _ptr(gradOutput),
+                                             _ptr(self.gradWeight), _ptr(self.gradBias),
+                                             ctypes.c_float(scale), _stream()))
+
+    def backward(self, input, gradOutput, scale=1.0):
+        self.updateGradInput(input, gradOutput)
+        self.accGradParameters(input, gradOutput, scale)
+        return self.gradInput
+
+    def cleanupBuffers(self):
+        for plan in self._plans.values():
+            plan.close()
+        self._plans = {}
+
+
+class SpatialConvolutionFBFFT(SpatialConvolutionFFT):
+    """nn.SpatialConvolutionFBFFT (fbcunn/SpatialConvolutionFBFFT.lua)."""
+    fftImplementation = "fbfft"
+
+
+class SpatialConvolutionFBFFTGemm(SpatialConvolutionFFT):
+    """nn.SpatialConvolutionFBFFTGemm (fbcunn/SpatialConvolutionFBFFTGemm.lua).  The
+    reference differs from FBFFT only in HOW the per-frequency contraction is
+    done (explicit transposes + cuBLAS Cgemm); here both modules share the one
+    frequency-major MFMA contraction, which is the layout that variant builds."""
+    fftImplementation = "fbfft"
+
+
+class FFTWrapper:
+    """nn.FFTWrapper with the fbfft backend (fbcunn/FFTWrapper.lua:53-132).
+
+    fft(time, frequency): time (..., h, w) real; frequency is frequency-major:
+    a float tensor of shape (N, N/2+1, planes, 2).  ffti is unnormalised."""
+
+    def __init__(self, cufft=None, padLeft=0, padUp=0, timed=False):
+        if cufft not in (None, "fbfft", False, 0):
+            raise ValueError("only the fbfft implementation exists in this build")
+        self.padLeft, self.padUp = padLeft, padUp
+        self.timed = timed
+
+    @staticmethod
+    def _dims(time, frequency):
+        _check_tensor(time, "time")
+        _check_tensor(frequency, "frequency", 4)
+        n = frequency.size(0)
+        planes = frequency.size(2)
+        if frequency.size(1) != n // 2 + 1 or frequency.size(3) != 2:
+            raise ValueError("frequency must be (N, N/2+1, planes, 2)")
+        h, w = time.size(-2), time.size(-1)
+        if time.numel() != planes * h * w:
+            raise ValueError("time and frequency disagree on the number of planes")
+        return n, planes, h, w
+
+    def fft(self, time, frequency, batchDims=None):
+        n, planes, h, w = self._dims(time, frequency)
+        check(lib().fbfc_fft2d(_ptr(time), planes, h, w, self.padUp, self.padLeft, n,
+                               _ptr(frequency), _stream()))
+        return frequency
+
+    def ffti(self, time, frequency, batchDims=None, bias=None):
+        n, planes, h, w = self._dims(time, frequency)
+        period = bias.numel() if bias is not None else 1
+        check(lib().fbfc_ifft2d(_ptr(frequency), planes, h, w, self.padUp, self.padLeft, n,
+                                _ptr(time), _ptr(bias), period, _stream()))
+        return time
+
+
+def transposeMM(A, B, C, invNorm, conjugateTransposeA, conjugateTransposeB, accumulate):
+    """transposeMMFFI (src/MM.cu:54-73) on frequency-major operands (Q, rows, cols, 2)."""
+    for t, nme in ((A, "A"), (B, "B"), (C, "C")):
+        _check_tensor(t, nme, 4)
+    Q, m, n = C.size(0), C.size(1), C.size(2)
+    k = A.size(1) if conjugateTransposeA else A.size(2)
+    exp_a = (Q, k, m, 2) if conjugateTransposeA else (Q, m, k, 2)
+    exp_b = (Q, n, k, 2) if conjugateTransposeB else (Q, k, n, 2)
+    if tuple(A.shape) != exp_a or tuple(B.shape) != exp_b:
+        raise ValueError("operand shapes do not match: A %s B %s C %s" % (tuple(A.shape), tuple(B.shape), tuple(C.shape)))
+    check(lib().fbfc_transpose_mm(_ptr(A), _ptr(B), _ptr(C), Q, m, n, k, ctypes.c_float(invNorm),
+                                  int(bool(conjugateTransposeA)), int(bool(conjugateTransposeB)),
+                                  int(bool(accumulate)), _stream()))
+    return C
+
+
+def updateOutputBias(output, bias):
+    """updateOutputBiasFFI (src/ConvolutionBias.cu:256-260)."""
+    _check_tensor(output, "output", 4)
+    _check_tensor(bias, "bias", 1)
+    B, F, h, w = output.shape
+    check(lib().fbfc_update_output_bias(_ptr(output), _ptr(bias), B, F, h, w, _stream()))
+    return output
+
+
+def accGradParametersBias(gradOutput, gradBias, scale=1.0):
+    """accGradParametersBiasFFI (src/ConvolutionBias.cu:262-274): gradBias is assigned."""
+    _check_tensor(gradOutput, "gradOutput", 4)
+    _check_tensor(gradBias, "gradBias", 1)
+    B, F, h, w = gradOutput.shape
+    nbytes = lib().fbfc_bias_grad_scratch_bytes(B, F)
+    scratch = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=gradOutput.device)
+    check(lib().fbfc_acc_grad_parameters_bias(_ptr(gradOutput), _ptr(gradBias), ctypes.c_float(scale),
+                                              B, F, h, w, _ptr(scratch), _stream()))
+    return gradBias

@@ -1,0 +1,170 @@
+/*
+ * fbfftconv — C ABI of the MI355X (gfx950) FFT-convolution library.
+ *
+ * This is the boundary a host binding loads (LuaJIT ffi.load, ctypes, dlopen).
+ * Every entry point takes plain device pointers, sizes and an opaque
+ * hipStream_t (passed as void*); there are no torch/THC types.  Every entry
+ * point returns FBFC_OK or an error code and never throws; the message for the
+ * last error on the calling thread is fbfc_last_error().
+ *
+ * Tensors are contiguous fp32, NCHW.  "planes" of a 4-D tensor (d0,d1,h,w) means
+ * the d0*d1 flattened leading dimensions.
+ *
+ * Frequency-domain buffers are FREQUENCY-MAJOR, complex interleaved:
+ *     freq[(ky * (N/2+1) + kx) * planes + plane] = (re, im)
+ * with ky in [0,N) the row frequency, kx in [0,N/2] the (Hermitian-halved)
+ * column frequency.  For a fixed frequency the planes form a dense row-major
+ * (d0 x d1) complex matrix, which is what the per-frequency contraction reads.
+ */
+#ifndef FBFFTCONV_H
+#define FBFFTCONV_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Error codes.  UNSUPPORTED_SIZE / UNSUPPORTED_DIMENSION mirror
+ * FBFFTParameters::ErrorCode as used in src/fft/FBFFTHost.cpp:96-98,115,168. */
+enum {
+    FBFC_OK = 0,
+    FBFC_ERR_INVALID_ARGUMENT = 1,
+    FBFC_ERR_UNSUPPORTED_SIZE = 2,
+    FBFC_ERR_UNSUPPORTED_DIMENSION = 3,
+    FBFC_ERR_OUT_OF_MEMORY = 4,
+    FBFC_ERR_HIP = 5
+};
+
+/* Constructor arguments of nn.SpatialConvolutionFBFFT
+ * (fbcunn/SpatialConvolutionFBFFT.lua:26-96, fbcunn/SpatialConvolutionFFT.lua:150-177)
+ * plus the batch and input size the reference only learns at the first call. */
+typedef struct {
+    int batch;      /* B */
+    int in_planes;  /* nInputPlane  P */
+    int out_planes; /* nOutputPlane F */
+    int in_h, in_w; /* H, W */
+    int k_h, k_w;   /* kH, kW */
+    int stride_h, stride_w; /* dH, dW: must be 1 */
+    int pad_h, pad_w;       /* padUp (= padDown), padLeft (= padRight): must be < kernel */
+} fbfc_conv_desc;
+
+/* What the reference derives in prepareFBFFTSizeAndBuffers
+ * (fbcunn/SpatialConvolutionFFT.lua:947-964) and getBuffer (:692-803). */
+typedef struct {
+    int fft_size;        /* N: smallest 2^i >= max(H+2padH, W+2padW, kH, kW, oH, oW), i >= 1 */
+    int n_freq;          /* Q = N * (N/2+1) */
+    int out_h, out_w;    /* H + 2 padH - kH + 1, W + 2 padW - kW + 1 */
+    size_t input_freq_bytes;   /* Q * B * P * 8 */
+    size_t weight_freq_bytes;  /* Q * F * P * 8 */
+    size_t output_freq_bytes;  /* Q * B * F * 8 */
+    size_t scratch_bytes;      /* bias-gradient partial sums */
+} fbfc_plan_info;
+
+typedef struct fbfc_plan fbfc_plan;
+
+/* Library ------------------------------------------------------------------ */
+const char *fbfc_version(void);
+/* Message of the last failure on this thread ("" if none). */
+const char *fbfc_last_error(void);
+
+/* Planning (host only; no GPU needed) ----------------------------------------
+ * Validates the descriptor the way the module constructor and the FFT-size
+ * choice do (stride 1: SpatialConvolutionFFT.lua:176, SpatialConvolutionFBFFT.lua:60-61;
+ * pad < kernel: SpatialConvolutionFBFFT.lua:93-95; nextPowerOf2: SpatialConvolutionFFT.lua:875-882)
+ * and fills *info.  FFT sizes above 64 are FBFC_ERR_UNSUPPORTED_SIZE. */
+int fbfc_plan_query(const fbfc_conv_desc *desc, fbfc_plan_info *info);
+
+/* Plans -----------------------------------------------------------------------
+ * A plan owns the three frequency-domain buffers of one layer shape (the
+ * reference's inputBuffer / weightBuffer / outputBuffer,
+ * SpatialConvolutionFFT.lua:652-688) on the current device.  Caller tensors are
+ * never kept or freed.  Passes on one plan must not overlap in time. */
+int fbfc_plan_create(const fbfc_conv_desc *desc, fbfc_plan **plan);
+int fbfc_plan_destroy(fbfc_plan *plan);
+int fbfc_plan_get_info(const fbfc_plan *plan, fbfc_plan_info *info);
+
+/* Replaces SpatialConvolutionFBFFT:updateOutputFFTImpl
+ * (fbcunn/SpatialConvolutionFBFFT.lua:102-183):
+ * output(B,F,oH,oW) = valid cross-correlation of zero-padded input(B,P,H,W) with
+ * weight(F,P,kH,kW), plus bias(F) (bias may be NULL = the reference's skipBias). */
+int fbfc_update_output(fbfc_plan *plan, const float *input, const float *weight,
+                       const float *bias, float *output, void *stream);
+
+/* Replaces SpatialConvolutionFBFFT:updateGradInputFFTImpl (:189-263):
+ * grad_input(B,P,H,W) = full convolution of grad_output(B,F,oH,oW) with weight,
+ * cropped to the un-padded input window. */
+int fbfc_update_grad_input(fbfc_plan *plan, const float *grad_output, const float *weight,
+                           float *grad_input, void *stream);
+
+/* Replaces SpatialConvolutionFBFFT:accGradParametersFFTImpl (:269-354):
+ * grad_weight(F,P,kH,kW) = scale * sum_b input(b,p) cross-correlated with
+ * grad_output(b,f); grad_bias(F) = scale * sum grad_output.  Both are ASSIGNED
+ * (the reference passes accumulate=false and its bias kernel assigns,
+ * src/ConvolutionBias.cu:95).  grad_bias may be NULL (skipBias). */
+int fbfc_acc_grad_parameters(fbfc_plan *plan, const float *input, const float *grad_output,
+                             float *grad_weight, float *grad_bias, float scale, void *stream);
+
+/* Memory-reuse policy of the module (SpatialConvolutionFFT.lua:59-63,216-240;
+ * used at SpatialConvolutionFBFFT.lua:226-230,305-322): with a flag set, the
+ * pass that would recompute that spectrum reuses the one the previous pass left
+ * in the plan's buffer.  Default 0 = memoryReuseNone (every pass recomputes). */
+enum { FBFC_REUSE_NONE = 0, FBFC_REUSE_INPUT = 1, FBFC_REUSE_OUTPUT = 2, FBFC_REUSE_WEIGHT = 4,
+       FBFC_REUSE_ALL = 7 };
+int fbfc_plan_set_reuse(fbfc_plan *plan, unsigned flags);
+
+/* Per-stage timing, the counterpart of the `timed` flag of nn.FFTWrapper /
+ * nn.CuBLASWrapper (src/fft/FFTWrapperLua.cpp:82-177): when on, each pass
+ * brackets its kernels with HIP events on the pass's stream and synchronises at
+ * the end.  Stage slots: */
+enum { FBFC_STAGE_FFT_A = 0,   /* first forward FFT of the pass  */
+       FBFC_STAGE_FFT_B = 1,   /* second forward FFT of the pass */
+       FBFC_STAGE_MM = 2,      /* per-frequency contraction      */
+       FBFC_STAGE_IFFT = 3,    /* inverse FFT (+ bias)           */
+       FBFC_STAGE_BIAS_GRAD = 4,
+       FBFC_NUM_STAGES = 5 };
+int fbfc_plan_set_timed(fbfc_plan *plan, int on);
+/* Milliseconds of each stage of the last timed pass (0 for a stage not run). */
+int fbfc_plan_stage_ms(const fbfc_plan *plan, float *ms, int n);
+
+/* Stand-alone stages ------------------------------------------------------------
+ * Replaces FFTWrapper_fft with fbfft (src/fft/FFTWrapperLua.cpp:209-272 ->
+ * fbfft2dHost, src/fft/FBFFTHost.cpp:39-116): batched 2-D real-to-complex FFT of
+ * `planes` h x w planes, each implicitly zero-padded into an N x N canvas at
+ * row pad_u, column pad_l.  N in {8,16,32,64}.  Output is frequency-major. */
+int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l,
+               int fft_size, float *freq, void *stream);
+
+/* Replaces FFTWrapper_ffti (same files): UNNORMALISED complex-to-real inverse;
+ * writes real[plane][r][s] = y[r+pad_u][s+pad_l] for r<h, s<w of the N x N result.
+ * If bias != NULL, bias[plane % bias_period] is added to every element of the
+ * plane (the fused form of updateOutputBiasFFI, src/ConvolutionBias.cu:39-51). */
+int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l,
+                int fft_size, float *real, const float *bias, int bias_period, void *stream);
+
+/* Replaces transposeMMFFI (src/MM.cu:54-73): for each of n_freq frequencies,
+ *   C (m x n) (=|+=) inv_norm * op(A) * op(B),   op = conjugate transpose if flagged.
+ * A is (m x k), or (k x m) when conj_trans_a; B is (k x n), or (n x k) when
+ * conj_trans_b; all dense row-major complex, frequency-major
+ * (X[freq][row][col][2]).  Both flags set is not supported (the reference does
+ * not instantiate it either, src/MM.cu:34-39). */
+int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq,
+                      int m, int n, int k, float inv_norm,
+                      int conj_trans_a, int conj_trans_b, int accumulate, void *stream);
+
+/* Replaces updateOutputBiasFFI (src/ConvolutionBias.cu:256-260): output[b][f][.][.] += bias[f]. */
+int fbfc_update_output_bias(float *output, const float *bias, int batch, int planes,
+                            int h, int w, void *stream);
+
+/* Replaces accGradParametersBiasFFI (src/ConvolutionBias.cu:262-274):
+ * grad_bias[f] = scale * sum_{b,r,c} grad_output[b][f][r][c] (assignment).
+ * scratch must hold fbfc_bias_grad_scratch_bytes(batch, planes) bytes. */
+size_t fbfc_bias_grad_scratch_bytes(int batch, int planes);
+int fbfc_acc_grad_parameters_bias(const float *grad_output, float *grad_bias, float scale,
+                                  int batch, int planes, int h, int w,
+                                  float *scratch, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FBFFTCONV_H */

@@ -1,0 +1,74 @@
+"""CPU-only checks of the shipped library: it loads, exports every symbol the
+header declares, and its host-side planning follows the reference's rules.  No
+compute entry point is called here."""
+import os
+import re
+
+import pytest
+
+from fbcunn_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "fbfftconv.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(fbfc_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 18
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    handle = _lib.lib()                       # raises if the .so is missing
+    for name in declared:
+        assert hasattr(handle, name), name
+    assert b"gfx950" in handle.fbfc_version()
+
+
+def _q(**kw):
+    base = dict(batch=2, in_planes=3, out_planes=4, in_h=13, in_w=13, k_h=3, k_w=3,
+                stride_h=1, stride_w=1, pad_h=1, pad_w=1)
+    base.update(kw)
+    return _lib.plan_query(**base)
+
+
+# FFT size = nextPowerOf2(max(H+2pU, W+2pL, kH, kW, oH, oW)), fbcunn/SpatialConvolutionFFT.lua:947-956
+@pytest.mark.parametrize("kw,n,q,o", [
+    (dict(batch=128, in_planes=64, out_planes=64, in_h=27, in_w=27, k_h=5, k_w=5, pad_h=2, pad_w=2), 32, 544, 27),
+    (dict(batch=128, in_planes=128, out_planes=128, in_h=13, in_w=13, k_h=3, k_w=3, pad_h=1, pad_w=1), 16, 144, 13),
+    (dict(batch=64, in_planes=96, out_planes=256, in_h=55, in_w=55, k_h=9, k_w=9, pad_h=4, pad_w=4), 64, 2112, 55),
+    (dict(batch=4, in_planes=16, out_planes=16, in_h=32, in_w=32, k_h=5, k_w=5, pad_h=0, pad_w=0), 32, 544, 28),
+    (dict(in_h=3, in_w=3, k_h=2, k_w=2, pad_h=0, pad_w=0), 8, 40, 2),      # tiny: canvas rounded up to 8
+    (dict(in_h=16, in_w=9, k_h=3, k_w=3, pad_h=1, pad_w=0), 32, 544, 16),   # square canvas from the larger side
+])
+def test_plan_sizes(kw, n, q, o):
+    info = _q(**kw)
+    assert (info.fft_size, info.n_freq, info.out_h) == (n, q, o)
+
+
+def test_plan_buffer_bytes_match_reference_layout():
+    # (d0, d1, N/2+1, N, 2) floats per buffer, fbcunn/SpatialConvolutionFFT.lua:710-721
+    info = _q(batch=128, in_planes=64, out_planes=64, in_h=27, in_w=27, k_h=5, k_w=5, pad_h=2, pad_w=2)
+    assert info.input_freq_bytes == 128 * 64 * 17 * 32 * 2 * 4
+    assert info.weight_freq_bytes == 64 * 64 * 17 * 32 * 2 * 4
+    assert info.output_freq_bytes == 128 * 64 * 17 * 32 * 2 * 4
+
+
+@pytest.mark.parametrize("kw,code,text", [
+    (dict(stride_h=2), _lib.ERR_INVALID_ARGUMENT, "stride-1"),
+    (dict(stride_w=3), _lib.ERR_INVALID_ARGUMENT, "stride-1"),
+    (dict(pad_h=3), _lib.ERR_INVALID_ARGUMENT, "Padding must be smaller than kernel"),
+    (dict(pad_w=5), _lib.ERR_INVALID_ARGUMENT, "Padding must be smaller than kernel"),
+    (dict(batch=0), _lib.ERR_INVALID_ARGUMENT, "positive"),
+    (dict(in_h=2, in_w=2, k_h=5, k_w=5, pad_h=0, pad_w=0), _lib.ERR_INVALID_ARGUMENT, "kernel larger"),
+    (dict(in_h=100, in_w=100), _lib.ERR_UNSUPPORTED_SIZE, "not supported"),
+    (dict(in_h=2000, in_w=5), _lib.ERR_UNSUPPORTED_SIZE, "Too large"),
+])
+def test_plan_rejections(kw, code, text):
+    with pytest.raises(_lib.FbfcError) as e:
+        _q(**kw)
+    assert e.value.code == code
+    assert text in e.value.message
+
+
+def test_scratch_size_query():
+    assert _lib.lib().fbfc_bias_grad_scratch_bytes(128, 64) >= 64 * 4
+    assert _lib.lib().fbfc_bias_grad_scratch_bytes(0, 64) == 0

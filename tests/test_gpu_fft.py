@@ -1,0 +1,140 @@
+"""GPU parity of the batched 2-D real<->complex FFT kernels, called through the
+C ABI (fbfc_fft2d / fbfc_ifft2d via nn.FFTWrapper), against the oracle's naive
+DFT on sampled planes and numpy.fft on all planes (the oracle's DFT is itself
+pinned against numpy.fft and the reference's cuFFT vectors in
+tests/test_oracle_fft.py).
+
+Tolerance: |err| <= 5e-6 * max|expected| (the reference compares fbfft with cuFFT
+at 4e-7 * max per element for sizes up to 128, test/test_FFTModule.lua:13; the
+sums here have up to 4096 float32 terms).
+"""
+import numpy as np
+import pytest
+import torch
+
+from fbcunn_amd import synth
+from gpu_util import dev, freq_major_to_planes, host, planes_to_freq_major
+
+pytestmark = pytest.mark.gpu
+TOL = 5e-6
+
+
+@pytest.fixture(scope="module")
+def nn():
+    from fbcunn_amd import nn as mod
+    return mod
+
+
+CASES = [
+    # N, planes, h, w, padU, padL
+    (8, 5, 8, 8, 0, 0), (8, 130, 3, 3, 0, 0), (8, 64, 5, 6, 2, 1),
+    (16, 7, 13, 13, 1, 1), (16, 96, 16, 16, 0, 0), (16, 33, 3, 3, 0, 0), (16, 40, 10, 12, 3, 2),
+    (32, 3, 27, 27, 2, 2), (32, 48, 32, 32, 0, 0), (32, 17, 5, 5, 0, 0), (32, 35, 20, 28, 5, 1),
+    (64, 9, 55, 55, 4, 4), (64, 16, 64, 64, 0, 0), (64, 5, 9, 9, 0, 0), (64, 11, 33, 40, 7, 10),
+]
+
+
+def _canvas(x, n, pu, pl):
+    c = np.zeros((x.shape[0], n, n))
+    c[:, pu:pu + x.shape[1], pl:pl + x.shape[2]] = x
+    return c
+
+
+@pytest.mark.parametrize("n,planes,h,w,pu,pl", CASES)
+def test_forward_matches_dft(nn, oracle, n, planes, h, w, pu, pl):
+    x = synth.uniform(100 + n, (planes, h, w))
+    freq = torch.full((n, n // 2 + 1, planes, 2), float("nan"), device="cuda")
+    nn.FFTWrapper("fbfft", pl, pu).fft(dev(x), freq)
+    got = freq_major_to_planes(host(freq))
+    want = np.fft.rfft2(_canvas(x, n, pu, pl))
+    scale = np.abs(want).max()
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL * scale
+    # oracle's naive DFT on a few planes (first, last = ragged tail of the last workgroup)
+    pick = sorted({0, planes // 2, planes - 1})
+    o = oracle.dft2d_r2c(x[pick], n, n, pu, pl)
+    oc = o[..., 0] + 1j * o[..., 1]
+    assert np.abs(got[pick] - oc).max() <= TOL * scale
+    # columns 0 and N/2 of a real signal's spectrum are Hermitian in the row frequency
+    for v in (0, n // 2):
+        assert np.abs(got[:, 1:, v] - np.conj(got[:, :0:-1, v])).max() <= TOL * scale
+
+
+@pytest.mark.parametrize("n,planes,h,w,pu,pl", CASES)
+def test_inverse_matches_idft(nn, oracle, n, planes, h, w, pu, pl):
+    full = synth.uniform(200 + n, (planes, n, n))
+    spec = np.fft.rfft2(full.astype(np.float64))
+    freq = dev(planes_to_freq_major(spec))
+    out = torch.full((planes, h, w), float("nan"), device="cuda")
+    nn.FFTWrapper("fbfft", pl, pu).ffti(out, freq)
+    got = host(out)
+    want = full[:, pu:pu + h, pl:pl + w].astype(np.float64) * (n * n)   # unnormalised inverse
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL * np.abs(want).max() * 4
+    pick = sorted({0, planes - 1})
+    sp32 = np.stack([spec.real, spec.imag], -1).astype(np.float32)[pick]
+    o = oracle.idft2d_c2r(sp32, h, w, n, pu, pl)
+    assert np.abs(got[pick] - o).max() <= TOL * np.abs(want).max() * 4
+
+
+def test_inverse_adds_bias_per_plane(nn):
+    n, B, F, h = 16, 3, 5, 13
+    full = synth.uniform(31, (B * F, n, n))
+    freq = dev(planes_to_freq_major(np.fft.rfft2(full.astype(np.float64))))
+    bias = synth.uniform(32, (F,), -0.1, 0.1)
+    plain = torch.empty((B * F, h, h), device="cuda")
+    biased = torch.empty((B * F, h, h), device="cuda")
+    w = nn.FFTWrapper("fbfft")
+    w.ffti(plain, freq)
+    w.ffti(biased, freq, bias=dev(bias))
+    want = host(plain).reshape(B, F, h, h) + bias[None, :, None, None]
+    np.testing.assert_allclose(host(biased).reshape(B, F, h, h), want, rtol=0, atol=1e-4)
+
+
+def test_linearity_and_shift(nn):
+    """FFT(a x + b y) = a FFT(x) + b FFT(y); moving the plane by (padU, padL)
+    multiplies the spectrum by the shift phase."""
+    n, planes, h = 32, 20, 20
+    x, y = synth.uniform(41, (planes, h, h)), synth.uniform(42, (planes, h, h))
+    f = lambda a, pu=0, pl=0: host(nn.FFTWrapper("fbfft", pl, pu).fft(
+        dev(a), torch.empty((n, n // 2 + 1, planes, 2), device="cuda")))
+    fx, fy, fz = f(x), f(y), f((2 * x - 3 * y).astype(np.float32))
+    scale = np.abs(fz).max()
+    assert np.abs(fz - (2 * fx - 3 * fy)).max() <= 1e-5 * scale
+    pu, pl = 5, 9
+    shifted = freq_major_to_planes(f(x, pu, pl))
+    ky = np.arange(n)[:, None]
+    kx = np.arange(n // 2 + 1)[None, :]
+    phase = np.exp(-2j * np.pi * (ky * pu + kx * pl) / n)
+    assert np.abs(shifted - freq_major_to_planes(fx) * phase).max() <= 1e-5 * scale
+
+
+def test_config2_round_trip_8192_planes(nn, oracle):
+    """8192 planes of 32x32: IFFT(FFT(x)) / 1024 reproduces x, and the forward
+    transform matches the naive DFT on 64 sampled planes."""
+    n, planes = 32, 8192
+    x = synth.uniform(1002, (planes, n, n))
+    xd = dev(x)
+    freq = torch.empty((n, n // 2 + 1, planes, 2), device="cuda")
+    back = torch.empty((planes, n, n), device="cuda")
+    w = nn.FFTWrapper("fbfft")
+    w.fft(xd, freq)
+    w.ffti(back, freq)
+    err = float((back / (n * n) - xd).abs().max())
+    assert err <= 1e-5 * float(np.abs(x).max())
+    pick = np.linspace(0, planes - 1, 64).astype(int)
+    got = host(freq[:, :, torch.from_numpy(pick).cuda(), :])
+    got = freq_major_to_planes(got)
+    o = oracle.dft2d_r2c(x[pick], n, n)
+    oc = o[..., 0] + 1j * o[..., 1]
+    assert np.abs(got - oc).max() <= TOL * np.abs(oc).max()
+
+
+def test_fft_argument_errors(nn):
+    x = torch.zeros((4, 20, 20), device="cuda")
+    with pytest.raises(nn.FbfcError) as e:          # plane + pad does not fit
+        nn.FFTWrapper("fbfft", 0, 15).fft(x, torch.empty((32, 17, 4, 2), device="cuda"))
+    assert "fit" in e.value.message
+    with pytest.raises(nn.FbfcError) as e:          # unsupported size, like fbfft's error code
+        nn.FFTWrapper("fbfft").fft(x, torch.empty((24, 13, 4, 2), device="cuda"))
+    assert e.value.code == 2

@@ -1,0 +1,93 @@
+"""GPU parity of the per-frequency complex contraction (fbfc_transpose_mm, the
+replacement of transposeMMFFI) against the oracle's frequency-domain triple loop
+and numpy einsum, for the three conjugation modes the reference uses, ragged
+sizes and the accumulate flag.  Tolerance 2e-5 * max|expected| (float32 MFMA
+accumulation of up to 256 products)."""
+import numpy as np
+import pytest
+import torch
+
+from fbcunn_amd import synth
+from gpu_util import dev, host
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-5
+
+
+@pytest.fixture(scope="module")
+def nn():
+    from fbcunn_amd import nn as mod
+    return mod
+
+
+def _c(a):
+    return a[..., 0].astype(np.float64) + 1j * a[..., 1].astype(np.float64)
+
+
+SHAPES = [  # Q, m, n, k
+    (5, 64, 64, 16), (3, 128, 64, 64), (4, 32, 32, 32), (7, 1, 1, 1), (6, 3, 5, 7),
+    (2, 65, 33, 17), (3, 70, 130, 40), (2, 64, 256, 96), (9, 16, 16, 4), (2, 100, 20, 129),
+]
+
+
+@pytest.mark.parametrize("Q,m,n,k", SHAPES)
+@pytest.mark.parametrize("mode", ["fprop", "bprop", "accgrad"])
+def test_transpose_mm(nn, mode, Q, m, n, k):
+    ca, cb = (mode == "accgrad"), (mode == "fprop")
+    A = synth.uniform(1, (Q, k, m, 2) if ca else (Q, m, k, 2))
+    B = synth.uniform(2, (Q, n, k, 2) if cb else (Q, k, n, 2))
+    C = torch.full((Q, m, n, 2), float("nan"), device="cuda")
+    nn.transposeMM(dev(A), dev(B), C, 0.25, ca, cb, False)
+    got = _c(host(C))
+    a, b = _c(A), _c(B)
+    if mode == "fprop":
+        want = 0.25 * np.einsum("qmk,qnk->qmn", a, np.conj(b))
+    elif mode == "bprop":
+        want = 0.25 * np.einsum("qmk,qkn->qmn", a, b)
+    else:
+        want = 0.25 * np.einsum("qkm,qkn->qmn", np.conj(a), b)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL * np.abs(want).max()
+
+
+def test_accumulate_flag(nn):
+    Q, m, n, k = 3, 40, 50, 20
+    A, B = synth.uniform(3, (Q, m, k, 2)), synth.uniform(4, (Q, k, n, 2))
+    C0 = synth.uniform(5, (Q, m, n, 2))
+    C = dev(C0)
+    nn.transposeMM(dev(A), dev(B), C, 1.0, False, False, True)
+    want = _c(C0) + np.einsum("qmk,qkn->qmn", _c(A), _c(B))
+    assert np.abs(_c(host(C)) - want).max() <= TOL * np.abs(want).max()
+
+
+@pytest.mark.parametrize("pass_", [0, 1, 2])
+def test_against_oracle_contraction(nn, oracle, pass_):
+    """Same numbers as the oracle's restatement of the reference's one-thread
+    frequency-domain kernels, after moving from plane-major to frequency-major."""
+    nB, nP, nF, Q = 6, 5, 4, 12
+    to_fm = lambda x: np.ascontiguousarray(np.transpose(x, (2, 0, 1, 3)))   # (d0,d1,Q,2) -> (Q,d0,d1,2)
+    I = synth.uniform(6, (nB, nP, Q, 2))
+    W = synth.uniform(7, (nF, nP, Q, 2))
+    G = synth.uniform(8, (nB, nF, Q, 2))
+    alpha = 1.0 / 64
+    if pass_ == 0:
+        want = oracle.freq_contract(0, I, W, nB, nP, nF, alpha)
+        C = torch.empty((Q, nB, nF, 2), device="cuda")
+        nn.transposeMM(dev(to_fm(I)), dev(to_fm(W)), C, alpha, False, True, False)
+    elif pass_ == 1:
+        want = oracle.freq_contract(1, G, W, nB, nP, nF, alpha)
+        C = torch.empty((Q, nB, nP, 2), device="cuda")
+        nn.transposeMM(dev(to_fm(G)), dev(to_fm(W)), C, alpha, False, False, False)
+    else:
+        want = oracle.freq_contract(2, G, I, nB, nP, nF, alpha)
+        C = torch.empty((Q, nF, nP, 2), device="cuda")
+        nn.transposeMM(dev(to_fm(G)), dev(to_fm(I)), C, alpha, True, False, False)
+    got = np.transpose(host(C), (1, 2, 0, 3))
+    assert np.abs(got - want).max() <= TOL * np.abs(want).max()
+
+
+def test_both_conjugations_rejected(nn):
+    t = torch.zeros((1, 2, 2, 2), device="cuda")
+    with pytest.raises(nn.FbfcError) as e:
+        nn.transposeMM(t, t, t.clone(), 1.0, True, True, False)
+    assert e.value.code == 3
