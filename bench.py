@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Benchmark of the FFT-convolution path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all-configs] [--no-cpu]
+
+One "step" is one full layer training step of the batch-128 configuration
+(updateOutput + updateGradInput + accGradParameters on batch 128, 128 -> 128
+planes, 13x13 input, 3x3 kernel, pad 1, FFT size 16) on synthetic inputs that are
+resident in HBM before the timed region starts.  `value` is the effective
+convolution rate: direct-convolution FLOPs (2*B*F*P*oH*oW*kH*kW per pass, three
+passes per step) divided by wall time.  The line also carries ms per pass, the
+roofline position of every stage (HIP events recorded by the library on the
+stream its kernels run on), the dominant kernel's roofline object and the CPU
+oracle timed on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_FP32_PEAK_TF = 157.3    # MI355X dense fp32 matrix, published
+
+CONFIGS = {
+    # name: B, P, F, H(=W), k, pad, passes, weight std, seed
+    "config3_fprop_b128_64x64_27x27_k5_p2": (128, 64, 64, 27, 5, 2, ("fprop",), 0.05, 1003),
+    "config4_step_b128_128x128_13x13_k3_p1": (128, 128, 128, 13, 3, 1, ("fprop", "bprop", "accgrad"), 0.05, 1004),
+    "config5_step_b64_96x256_55x55_k9_p4": (64, 96, 256, 55, 9, 4, ("fprop", "bprop", "accgrad"), 0.02, 1005),
+}
+MAIN = "config4_step_b128_128x128_13x13_k3_p1"
+
+
+def stage_model(cfg, pass_, n, q):
+    """Algorithmic bytes / flops of each stage of one pass (intermediates counted
+    once written and once read; no scratch traffic)."""
+    B, P, F, H, k, pad = cfg[:6]
+    o = H + 2 * pad - k + 1
+    fft = lambda planes, h: 4 * planes * h * h + 8 * planes * q
+    mm_bytes = lambda m, nn_, kk: 8 * q * (m * kk + kk * nn_ + m * nn_)
+    mm_flops = lambda m, nn_, kk: 8 * q * m * nn_ * kk
+    if pass_ == "fprop":
+        return {"fft_a": ("hbm", fft(B * P, H)), "fft_b": ("hbm", fft(F * P, k)),
+                "mm": ("mfma", mm_flops(B, F, P), mm_bytes(B, F, P)),
+                "ifft": ("hbm", fft(B * F, o))}
+    if pass_ == "bprop":
+        return {"fft_a": ("hbm", fft(B * F, o)), "fft_b": ("hbm", fft(F * P, k)),
+                "mm": ("mfma", mm_flops(B, P, F), mm_bytes(B, P, F)),
+                "ifft": ("hbm", fft(B * P, H))}
+    return {"bias_grad": ("hbm", 4 * B * F * o * o),
+            "fft_a": ("hbm", fft(B * F, o)), "fft_b": ("hbm", fft(B * P, H)),
+            "mm": ("mfma", mm_flops(F, P, B), mm_bytes(F, P, B)),
+            "ifft": ("hbm", fft(F * P, k))}
+
+
+KERNEL_OF_STAGE = {"fft_a": "rfft2d_kernel", "fft_b": "rfft2d_kernel", "mm": "cgemm_freq_kernel",
+                   "ifft": "irfft2d_kernel", "bias_grad": "bias_grad_partial_kernel"}
+
+
+def make_layer(nn, torch, synth, cfg):
+    B, P, F, H, k, pad, _, wstd, seed = cfg
+    o = H + 2 * pad - k + 1
+    net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad)
+    net.weight.copy_(torch.from_numpy(synth.normal(seed, (F, P, k, k), 0.0, wstd, stream=1)).cuda())
+    net.bias.copy_(torch.from_numpy(synth.uniform(seed, (F,), -0.1, 0.1, stream=2)).cuda())
+    x = torch.from_numpy(synth.uniform(seed, (B, P, H, H), stream=0)).cuda()
+    g = torch.from_numpy(synth.uniform(seed, (B, F, o, o), stream=3)).cuda()
+    return net, x, g
+
+
+def run_pass(net, x, g, pass_):
+    if pass_ == "fprop":
+        net.updateOutput(x)
+    elif pass_ == "bprop":
+        net.updateGradInput(x, g)
+    else:
+        net.accGradParameters(x, g, 1.0)
+
+
+def time_loop(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def measure_config(nn, torch, synth, name, steps, warmup):
+    cfg = CONFIGS[name]
+    B, P, F, H, k, pad, passes = cfg[:7]
+    o = H + 2 * pad - k + 1
+    net, x, g = make_layer(nn, torch, synth, cfg)
+    flop_pass = 2.0 * B * F * P * o * o * k * k
+    res = {"passes": {}}
+    # whole step, untimed stages
+    net.timed = False
+    ms_step = time_loop(torch, lambda: [run_pass(net, x, g, p) for p in passes], steps, warmup)
+    res["ms_per_step"] = ms_step
+    res["effective_tflops"] = flop_pass * len(passes) / (ms_step * 1e-3) / 1e12
+    plan = net._plan_for(B, H, H)
+    n, q = plan.info.fft_size, plan.info.n_freq
+    for p in passes:
+        net.timed = False
+        ms = time_loop(torch, lambda: run_pass(net, x, g, p), steps, warmup)
+        entry = {"ms": ms, "effective_tflops": flop_pass / (ms * 1e-3) / 1e12, "stages": {}}
+        # per-stage HIP-event timing (the library records events on the pass's stream)
+        net.timed = True
+        acc = {}
+        reps = max(3, min(steps, 20))
+        run_pass(net, x, g, p)
+        for _ in range(reps):
+            run_pass(net, x, g, p)
+            for s, v in net.stageTimes(x).items():
+                acc[s] = acc.get(s, 0.0) + v
+        net.timed = False
+        model = stage_model(cfg, p, n, q)
+        for s, spec in model.items():
+            ms_s = acc.get(s, 0.0) / reps
+            if ms_s <= 0:
+                continue
+            if spec[0] == "hbm":
+                ach = spec[1] / (ms_s * 1e-3) / 1e9
+                entry["stages"][s] = {"kernel": KERNEL_OF_STAGE[s], "ms": ms_s, "bound": "hbm",
+                                      "bytes": spec[1], "achieved": ach, "unit": "GB/s",
+                                      "peak": HBM_PEAK_GBS, "frac": ach / HBM_PEAK_GBS}
+            else:
+                ach = spec[1] / (ms_s * 1e-3) / 1e12
+                entry["stages"][s] = {"kernel": KERNEL_OF_STAGE[s], "ms": ms_s, "bound": "mfma",
+                                      "flops": spec[1], "bytes": spec[2], "achieved": ach,
+                                      "unit": "TFLOP/s", "peak": MFMA_FP32_PEAK_TF,
+                                      "frac": ach / MFMA_FP32_PEAK_TF,
+                                      "hbm_gbs": spec[2] / (ms_s * 1e-3) / 1e9}
+        res["passes"][p] = entry
+    res["fft_size"] = n
+    net.cleanupBuffers()
+    return res
+
+
+def measure_fft_round_trip(nn, torch, synth, steps, warmup):
+    """8192 planes of 32x32: forward then inverse, each timed on its own."""
+    n, planes = 32, 8192
+    x = torch.from_numpy(synth.uniform(1002, (planes, n, n))).cuda()
+    freq = torch.empty((n, n // 2 + 1, planes, 2), device="cuda")
+    back = torch.empty_like(x)
+    w = nn.FFTWrapper("fbfft")
+    out = {}
+    for name, fn in (("fft", lambda: w.fft(x, freq)), ("ifft", lambda: w.ffti(back, freq))):
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(warmup):
+            fn()
+        ev0.record()
+        for _ in range(steps):
+            fn()
+        ev1.record()
+        torch.cuda.synchronize()
+        ms = ev0.elapsed_time(ev1) / steps
+        nbytes = 4 * planes * n * n + 8 * planes * n * (n // 2 + 1)
+        ach = nbytes / (ms * 1e-3) / 1e9
+        out[name] = {"ms": ms, "bytes": nbytes, "achieved": ach, "unit": "GB/s", "peak": HBM_PEAK_GBS,
+                     "frac": ach / HBM_PEAK_GBS}
+    return out
+
+
+def cpu_baseline(synth):
+    """The CPU oracle on the main workload: the whole batch-128 training step
+    (three passes, 19.1 GFLOP of direct convolution), all host threads OpenMP
+    gives it, one run after a small warm-up."""
+    import oracle
+    cfg = CONFIGS[MAIN]
+    B, P, F, H, k, pad, passes, wstd, seed = cfg
+    o = H + 2 * pad - k + 1
+    x = synth.uniform(seed, (B, P, H, H), stream=0)
+    w = synth.normal(seed, (F, P, k, k), 0.0, wstd, stream=1)
+    g = synth.uniform(seed, (B, F, o, o), stream=3)
+    p4 = (pad,) * 4
+    oracle.cross_correlation_valid(x[:2], w, (1, 1), p4)   # warm-up (loads the library, spins up threads)
+    t0 = time.perf_counter()
+    oracle.cross_correlation_valid(x, w, (1, 1), p4)
+    oracle.convolution_full(g, w, (1, 1), p4)
+    oracle.cross_correlation_reverse_valid(x, g, (1, 1), 1.0, p4)
+    dt = time.perf_counter() - t0
+    flops = 3 * 2.0 * B * F * P * o * o * k * k
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "ms_per_step": dt * 1e3,
+            "sample": "the whole %s step (fprop+bprop+accGrad, %.1f GFLOP), 1 run, OpenMP over independent outputs"
+                      % (MAIN, flops / 1e9)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--all-configs", action="store_true", help="also measure configs 2, 3 and 5")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives exist on this path); "
+                 "use --gpus 1")
+
+    import torch
+    from fbcunn_amd import nn, synth
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    torch.cuda.set_device(0)
+
+    main_res = measure_config(nn, torch, synth, MAIN, args.steps, args.warmup)
+    # dominant kernel of the step = the stage with the largest summed time
+    worst, worst_ms = None, -1.0
+    for p, e in main_res["passes"].items():
+        for s, st in e["stages"].items():
+            if st["ms"] > worst_ms:
+                worst, worst_ms = (p, s, st), st["ms"]
+    p, s, st = worst
+    roofline = {"bound": st["bound"], "achieved": st["achieved"], "peak": st["peak"], "unit": st["unit"],
+                "frac": st["frac"], "traffic": None, "kernel": st["kernel"], "pass": p, "stage": s,
+                "avg_launch_ms": st["ms"]}
+
+    line = {
+        "metric": "effective conv TFLOP/s (direct-convolution FLOPs / time), full training step at batch 128",
+        "value": main_res["effective_tflops"], "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": MAIN, "fft_size": main_res["fft_size"],
+                   "step": "updateOutput+updateGradInput+accGradParameters, every pass recomputes its FFTs"},
+        "ms_per_pass": {k: v["ms"] for k, v in main_res["passes"].items()},
+        "tflops_per_pass": {k: v["effective_tflops"] for k, v in main_res["passes"].items()},
+        "roofline": roofline,
+        "stages": {k: v["stages"] for k, v in main_res["passes"].items()},
+    }
+    if args.all_configs:
+        others = {}
+        for name in CONFIGS:
+            if name != MAIN:
+                others[name] = measure_config(nn, torch, synth, name, max(5, args.steps // 5), 2)
+        others["config2_fft_round_trip_8192x32x32"] = measure_fft_round_trip(nn, torch, synth, args.steps, args.warmup)
+        line["other_configs"] = others
+    line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
