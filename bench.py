@@ -200,6 +200,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all-configs", action="store_true", help="also measure configs 2, 3 and 5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run a plain 256 MiB device copy 3 times (a kernel of known traffic "
+                         "for scaling FETCH_SIZE / WRITE_SIZE counter readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives exist on this path); "
@@ -210,6 +213,14 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     torch.cuda.set_device(0)
+
+    if args.calibrate_copy:
+        a = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
 
     main_res = measure_config(nn, torch, synth, MAIN, args.steps, args.warmup)
     # dominant kernel of the step = the stage with the largest summed time
