@@ -34,12 +34,17 @@ struct FftShape {
     static constexpr int THREADS = 256;     // T * N / 2
     static constexpr int NH2 = N / 2;       // complex slots per tile row
     static constexpr int NH = N / 2 + 1;    // stored column frequencies
+    // Phases: the LDS tile holds NH2/PH of the tile columns at a time and the input /
+    // output staging area T/PH planes at a time, so that two workgroups fit one CU's
+    // 160 KB LDS even for N = 64 (a full 8-plane tile would need 117 KB).
+    static constexpr int PH = (N >= 64) ? 2 : 1;
+    static constexpr int KXP = NH2 / PH;    // tile columns per phase
+    static constexpr int TP = T / PH;       // planes per staging round
     // padding (in complex elements) between tile rows: keeps the T-lane groups
     // of one wave on different LDS banks when T*8 bytes is below 128
     static constexpr int ROWPAD = (T * 8 < 128) ? (64 / 8) / 2 : 0;
-    static constexpr int ROWSTRIDE = NH2 * T + ROWPAD;  // complex elements
+    static constexpr int ROWSTRIDE = KXP * T + ROWPAD;  // complex elements
 };
-
 
 // Copies np whole planes of hw floats between a contiguous global chunk and an
 // LDS staging area whose plane stride hwp = hw|1 is odd, so that lanes reading
@@ -93,7 +98,7 @@ __device__ __forceinline__ void copy_planes(float *smem, float *g, int np, int h
 // forward: real (planes,h,w) -> freq [N*(N/2+1)][planes] complex
 // ---------------------------------------------------------------------------------
 template <int N>
-__global__ __launch_bounds__(256) void rfft2d_kernel(const float *__restrict__ in,
+__global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(const float *__restrict__ in,
                                                      float2 *__restrict__ out, long planes,
                                                      int h, int w, int padU, int padL, int vec4)
 {
@@ -108,10 +113,6 @@ __global__ __launch_bounds__(256) void rfft2d_kernel(const float *__restrict__ i
     const int y_lo = padU & ~1;                       // first canvas row that can be non-zero (even)
     const int y_hi = (padU + h + 1) & ~1;             // one past the last, rounded up to even
 
-    // ---- stage the contiguous chunk of np planes ----
-    copy_planes<true>(smem, const_cast<float *>(in) + x0 * hw, np, hw, hwp, vec4, tid);
-    __syncthreads();
-
     const int t = tid % T;
     float re[N], im[N];
 
@@ -122,24 +123,39 @@ __global__ __launch_bounds__(256) void rfft2d_kernel(const float *__restrict__ i
     const bool va = (ia >= 0) && (ia < h);
     const bool vb = (ib >= 0) && (ib < h);
     const bool row_active = (t < np) && (va || vb);
-    if (row_active) {
-        const float *pa = smem + t * hwp + ia * w - padL;
-        const float *pb = smem + t * hwp + ib * w - padL;
-        static_for<N>([&](auto cc) {
-            constexpr int c = decltype(cc)::value;
-            const bool vc = (c >= padL) && (c < padL + w);
-            re[c] = (va && vc) ? pa[c] : 0.0f;
-            im[c] = (vb && vc) ? pb[c] : 0.0f;
-        });
-    }
-    __syncthreads();  // staging chunk fully consumed; the tile may overwrite it
 
+    // ---- stage the contiguous chunk of planes, TP planes per round ----
+    static_for<S::PH>([&](auto hh) {
+        constexpr int hs = decltype(hh)::value;
+        int nph = np - hs * S::TP;
+        nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
+        if (hs > 0) __syncthreads();  // previous round fully read
+        copy_planes<true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph, hw, hwp, vec4, tid);
+        __syncthreads();
+        if (row_active && (t / S::TP) == hs) {
+            const float *pa = smem + (t - hs * S::TP) * hwp + ia * w - padL;
+            const float *pb = smem + (t - hs * S::TP) * hwp + ib * w - padL;
+            static_for<N>([&](auto cc) {
+                constexpr int c = decltype(cc)::value;
+                const bool vc = (c >= padL) && (c < padL + w);
+                re[c] = (va && vc) ? pa[c] : 0.0f;
+                im[c] = (vb && vc) ? pb[c] : 0.0f;
+            });
+        }
+    });
+
+    // ---- row FFT and untangling ----
+    // A[k] / B[k]: spectra of rows ya / yb; slot 0 carries the real-valued columns 0 and N/2.
+    // The first phase's columns go straight to the LDS tile, later ones wait in registers.
+    constexpr int NLATE = S::NH2 - S::KXP;  // 0 when there is a single phase
+    float ar[NLATE > 0 ? NLATE : 1], ai[NLATE > 0 ? NLATE : 1], br[NLATE > 0 ? NLATE : 1], bi[NLATE > 0 ? NLATE : 1];
     float2 *R = reinterpret_cast<float2 *>(smem);
+    const int kx = tid / T;  // column pass: lane (t, kx) owns tile column kx of plane t
+    __syncthreads();  // staging area fully consumed; the tile may overwrite it
     if (row_active) {
         fft_inplace<N, false>(re, im);
         float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
         float2 *Rb = Ra + S::ROWSTRIDE;
-        // slot 0 carries the two real-valued columns 0 and N/2
         Ra[0] = make_float2(re[brev<N>(0)], re[brev<N>(N / 2)]);
         Rb[0] = make_float2(im[brev<N>(0)], im[brev<N>(N / 2)]);
         static_for<N / 2 - 1>([&](auto kk) {
@@ -147,23 +163,49 @@ __global__ __launch_bounds__(256) void rfft2d_kernel(const float *__restrict__ i
             const float zr = re[brev<N>(k)], zi = im[brev<N>(k)];
             const float nr = re[brev<N>(N - k)], ni = im[brev<N>(N - k)];
             // A = (Z[k] + conj Z[N-k]) / 2 ; B = -i (Z[k] - conj Z[N-k]) / 2
-            Ra[k * T] = make_float2(0.5f * (zr + nr), 0.5f * (zi - ni));
-            Rb[k * T] = make_float2(0.5f * (zi + ni), 0.5f * (nr - zr));
+            if constexpr (k < S::KXP) {
+                Ra[k * T] = make_float2(0.5f * (zr + nr), 0.5f * (zi - ni));
+                Rb[k * T] = make_float2(0.5f * (zi + ni), 0.5f * (nr - zr));
+            } else {
+                ar[k - S::KXP] = 0.5f * (zr + nr);  ai[k - S::KXP] = 0.5f * (zi - ni);
+                br[k - S::KXP] = 0.5f * (zi + ni);  bi[k - S::KXP] = 0.5f * (nr - zr);
+            }
         });
     }
-    __syncthreads();
 
-    // ---- column pass: lane (t, kx) owns tile column kx of plane t ----
-    const int kx = tid / T;
+    // Each phase: (later phases first refill the tile from registers) then the lanes whose
+    // column belongs to the phase pull it into registers, which frees the tile again.
+    static_for<S::PH>([&](auto pp) {
+        constexpr int ph = decltype(pp)::value;
+        if constexpr (ph > 0) {
+            __syncthreads();  // previous phase's columns are in registers
+            if (row_active) {
+                float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
+                float2 *Rb = Ra + S::ROWSTRIDE;
+                static_for<S::KXP>([&](auto kk) {
+                    constexpr int kl = decltype(kk)::value;
+                    constexpr int k = ph * S::KXP + kl - S::KXP;
+                    Ra[kl * T] = make_float2(ar[k], ai[k]);
+                    Rb[kl * T] = make_float2(br[k], bi[k]);
+                });
+            }
+        }
+        __syncthreads();
+        if ((t < np) && (kx / S::KXP) == ph) {
+            const int kl = kx - ph * S::KXP;
+            static_for<N>([&](auto yy) {
+                constexpr int y = decltype(yy)::value;
+                const bool vy = (y >= y_lo) && (y < y_hi);
+                float2 v = make_float2(0.0f, 0.0f);
+                if (vy) v = R[(y - y_lo) * S::ROWSTRIDE + kl * T + t];
+                re[y] = v.x;
+                im[y] = v.y;
+            });
+        }
+    });
+
+    // ---- column FFT and frequency-major store, all lanes at once ----
     if (t < np) {
-        static_for<N>([&](auto yy) {
-            constexpr int y = decltype(yy)::value;
-            const bool vy = (y >= y_lo) && (y < y_hi);
-            float2 v = make_float2(0.0f, 0.0f);
-            if (vy) v = R[(y - y_lo) * S::ROWSTRIDE + kx * T + t];
-            re[y] = v.x;
-            im[y] = v.y;
-        });
         fft_inplace<N, false>(re, im);
         float2 *o = out + x0 + t;
         if (kx != 0) {
@@ -190,7 +232,7 @@ __global__ __launch_bounds__(256) void rfft2d_kernel(const float *__restrict__ i
 // real[r][s] = y[r+padU][s+padL] (+ bias[plane % bias_period])
 // ---------------------------------------------------------------------------------
 template <int N>
-__global__ __launch_bounds__(256) void irfft2d_kernel(const float2 *__restrict__ in,
+__global__ __launch_bounds__(256, FftShape<N>::PH) void irfft2d_kernel(const float2 *__restrict__ in,
                                                       float *__restrict__ out, long planes,
                                                       int h, int w, int padU, int padL,
                                                       const float *__restrict__ bias,
@@ -211,7 +253,7 @@ __global__ __launch_bounds__(256) void irfft2d_kernel(const float2 *__restrict__
     float re[N], im[N];
     float2 *R = reinterpret_cast<float2 *>(smem);
 
-    // ---- column pass ----
+    // ---- column pass: lane (t, kx) fetches its whole column and transforms it, all lanes at once ----
     const int kx = tid / T;
     if (t < np) {
         const float2 *src = in + x0 + t;
@@ -233,54 +275,73 @@ __global__ __launch_bounds__(256) void irfft2d_kernel(const float2 *__restrict__
             });
         }
         fft_inplace<N, true>(re, im);
-        static_for<N>([&](auto yy) {
-            constexpr int y = decltype(yy)::value;
-            if ((y >= y_lo) && (y < y_hi))
-                R[(y - y_lo) * S::ROWSTRIDE + kx * T + t] = make_float2(re[brev<N>(y)], im[brev<N>(y)]);
-        });
     }
-    __syncthreads();
 
-    // ---- row pass: lane (t, rp) rebuilds canvas rows 2rp, 2rp+1 ----
+    // ---- row pass bookkeeping: lane (t, rp) rebuilds canvas rows 2rp, 2rp+1 ----
     const int rp = tid / T;
     const int ya = 2 * rp, yb = ya + 1;
     const int ia = ya - padU, ib = yb - padU;
     const bool va = (ia >= 0) && (ia < h);
     const bool vb = (ib >= 0) && (ib < h);
     const bool row_active = (t < np) && (va || vb);
-    if (row_active) {
-        const float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
-        const float2 *Rb = Ra + S::ROWSTRIDE;
-        // Z[k] = Ya[k] + i Yb[k], k = 0..N-1, with Y[N-k] = conj Y[k]
-        const float2 a0 = Ra[0], b0 = Rb[0];
-        re[0] = a0.x;       im[0] = b0.x;              // k = 0   : both real
-        re[N / 2] = a0.y;   im[N / 2] = b0.y;          // k = N/2 : both real
-        static_for<N / 2 - 1>([&](auto kk) {
-            constexpr int k = decltype(kk)::value + 1;
-            const float2 a = Ra[k * T], b = Rb[k * T];
-            re[k] = a.x - b.y;      im[k] = a.y + b.x;
-            re[N - k] = a.x + b.y;  im[N - k] = b.x - a.y;
-        });
-    }
+    // Z[k] = Ya[k] + i Yb[k], k = 0..N-1, with Y[N-k] = conj Y[k]
+    float zr[N], zi[N];
+
+    static_for<S::PH>([&](auto pp) {
+        constexpr int ph = decltype(pp)::value;
+        if (ph > 0) __syncthreads();  // previous phase's tile fully read
+        if ((t < np) && (kx / S::KXP) == ph) {
+            const int kl = kx - ph * S::KXP;
+            static_for<N>([&](auto yy) {
+                constexpr int y = decltype(yy)::value;
+                if ((y >= y_lo) && (y < y_hi))
+                    R[(y - y_lo) * S::ROWSTRIDE + kl * T + t] = make_float2(re[brev<N>(y)], im[brev<N>(y)]);
+            });
+        }
+        __syncthreads();
+        if (row_active) {
+            const float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
+            const float2 *Rb = Ra + S::ROWSTRIDE;
+            static_for<S::KXP>([&](auto kk) {
+                constexpr int kl = decltype(kk)::value;
+                constexpr int k = ph * S::KXP + kl;
+                const float2 a = Ra[kl * T], b = Rb[kl * T];
+                if constexpr (k == 0) {
+                    zr[0] = a.x;      zi[0] = b.x;        // k = 0   : both real
+                    zr[N / 2] = a.y;  zi[N / 2] = b.y;    // k = N/2 : both real
+                } else {
+                    zr[k] = a.x - b.y;      zi[k] = a.y + b.x;
+                    zr[N - k] = a.x + b.y;  zi[N - k] = b.x - a.y;
+                }
+            });
+        }
+    });
     __syncthreads();  // tile fully consumed; the staging area may overwrite it
 
+    float bv = 0.0f;
     if (row_active) {
-        fft_inplace<N, true>(re, im);
-        float bv = 0.0f;
+        fft_inplace<N, true>(zr, zi);
         if (bias != nullptr) bv = bias[(x0 + t) % bias_period];
-        float *pa = smem + t * hwp + ia * w - padL;
-        float *pb = smem + t * hwp + ib * w - padL;
-        static_for<N>([&](auto cc) {
-            constexpr int c = decltype(cc)::value;
-            const bool vc = (c >= padL) && (c < padL + w);
-            if (va && vc) pa[c] = re[brev<N>(c)] + bv;
-            if (vb && vc) pb[c] = im[brev<N>(c)] + bv;
-        });
     }
-    __syncthreads();
-
-    // ---- coalesced copy-out ----
-    copy_planes<false>(smem, out + x0 * hw, np, hw, hwp, vec4, tid);
+    // ---- crop (+bias) into the staging area and coalesced copy-out, TP planes per round ----
+    static_for<S::PH>([&](auto hh) {
+        constexpr int hs = decltype(hh)::value;
+        int nph = np - hs * S::TP;
+        nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
+        if (hs > 0) __syncthreads();  // previous round copied out
+        if (row_active && (t / S::TP) == hs) {
+            float *pa = smem + (t - hs * S::TP) * hwp + ia * w - padL;
+            float *pb = smem + (t - hs * S::TP) * hwp + ib * w - padL;
+            static_for<N>([&](auto cc) {
+                constexpr int c = decltype(cc)::value;
+                const bool vc = (c >= padL) && (c < padL + w);
+                if (va && vc) pa[c] = zr[brev<N>(c)] + bv;
+                if (vb && vc) pb[c] = zi[brev<N>(c)] + bv;
+            });
+        }
+        __syncthreads();
+        copy_planes<false>(smem, out + (x0 + hs * S::TP) * hw, nph, hw, hwp, vec4, tid);
+    });
 }
 
 // ---------------------------------------------------------------------------------
@@ -294,7 +355,7 @@ static size_t fft_lds_bytes(int h, int w, int padU, bool inverse)
     const size_t tile = (size_t)(y_hi - y_lo) * S::ROWSTRIDE * sizeof(float2);
     (void)inverse;
     const size_t plane = (size_t)((h * w) | 1);
-    const size_t stage = (size_t)S::T * plane * sizeof(float);
+    const size_t stage = (size_t)S::TP * plane * sizeof(float);
     return ((tile > stage ? tile : stage) + 15) & ~(size_t)15;
 }
 
