@@ -46,52 +46,89 @@ struct FftShape {
     static constexpr int ROWSTRIDE = KXP * T + ROWPAD;  // complex elements
 };
 
-// Copies np whole planes of hw floats between a contiguous global chunk and an
-// LDS staging area whose plane stride hwp = hw|1 is odd, so that lanes reading
-// the same (row, column) of consecutive planes hit different banks.
-template <bool TO_LDS>
-__device__ __forceinline__ void copy_planes(float *smem, float *g, int np, int hw, int hwp,
+// LDS staging area in canvas-row layout.  Row (p*h + r) of the staged planes starts at
+// (p*h + r) * LDR floats and holds the N canvas columns of that row: input column x sits
+// at padL + x, the margins are zero.  LDR = N + 4 floats keeps rows 16-byte aligned (the
+// row pass reads and writes them with 16-byte LDS accesses) while rotating them over the
+// banks.  The global side is the contiguous chunk of nrows * w floats.
+template <int N>
+struct Canvas {
+    static constexpr int LDR = N + 4;
+};
+
+// Workgroup -> plane-group mapping.  Workgroups are handed to the 8 XCDs round-robin.  When a
+// group's run per frequency is only half a 128-byte line (T*8 = 64 bytes), the two groups that
+// share each line are given to workgroups b and b+8: same XCD, dispatched back to back, so the
+// two halves meet in that XCD's L2 (one line fetched once / written back whole).
+template <int N>
+__device__ __forceinline__ long plane_group(unsigned bid)
+{
+    if constexpr (FftShape<N>::T * 8 >= 128) {
+        return (long)bid;
+    } else {
+        const unsigned cyc = bid >> 4, r = bid & 15u;
+        return (long)(2u * (cyc * 8u + (r & 7u)) + (r >> 3));
+    }
+}
+
+template <int N, bool TO_LDS>
+__device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, int w, int padL,
                                             int vec4, int tid)
 {
-    const int total = np * hw;
-    if (vec4 && hwp == hw) {  // same layout on both sides: flat 16-byte copy
+    constexpr int LDR = Canvas<N>::LDR;
+    const int total = nrows * w;
+    int done = 0;
+    if (vec4) {
         const int n4 = total >> 2;
         float4 *g4 = reinterpret_cast<float4 *>(g);
-        float4 *s4 = reinterpret_cast<float4 *>(smem);
+        int row = (tid * 4) / w, x = tid * 4 - row * w;
+        const int drow = 1024 / w, dx = 1024 - drow * w;
         for (int i = tid; i < n4; i += 256) {
-            if (TO_LDS) s4[i] = g4[i]; else g4[i] = s4[i];
-        }
-        for (int i = (n4 << 2) + tid; i < total; i += 256) {
-            if (TO_LDS) smem[i] = g[i]; else g[i] = smem[i];
-        }
-    } else if (vec4 && (hw & 3) == 0) {  // 16-byte global accesses never straddle a plane
-        const int n4 = total >> 2;
-        float4 *g4 = reinterpret_cast<float4 *>(g);
-        int e = tid * 4;
-        int p = e / hw, off = e - p * hw;
-        const int dp = 1024 / hw, doff = 1024 - dp * hw;
-        for (int i = tid; i < n4; i += 256) {
-            float *s = smem + p * hwp + off;
+            float v[4];
             if (TO_LDS) {
-                const float4 v = g4[i];
-                s[0] = v.x; s[1] = v.y; s[2] = v.z; s[3] = v.w;
-            } else {
-                g4[i] = make_float4(s[0], s[1], s[2], s[3]);
+                const float4 q = g4[i];
+                v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
             }
-            p += dp;
-            off += doff;
-            if (off >= hw) { off -= hw; ++p; }
+            int r_ = row, x_ = x;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float *sp = smem + r_ * LDR + padL + x_;
+                if (TO_LDS) *sp = v[c]; else v[c] = *sp;
+                if (++x_ == w) { x_ = 0; ++r_; }
+            }
+            if (!TO_LDS) g4[i] = make_float4(v[0], v[1], v[2], v[3]);
+            row += drow;
+            x += dx;
+            if (x >= w) { x -= w; ++row; }
         }
-    } else {
-        int p = tid / hw, off = tid - p * hw;
-        const int dp = 256 / hw, doff = 256 - dp * hw;
-        for (int i = tid; i < total; i += 256) {
-            if (TO_LDS) smem[p * hwp + off] = g[i]; else g[i] = smem[p * hwp + off];
-            p += dp;
-            off += doff;
-            if (off >= hw) { off -= hw; ++p; }
+        done = n4 << 2;
+    }
+    {
+        const int first = done + tid;
+        int row = first / w, x = first - row * w;
+        const int drow = 256 / w, dx = 256 - drow * w;
+        for (int i = first; i < total; i += 256) {
+            float *sp = smem + row * LDR + padL + x;
+            if (TO_LDS) *sp = g[i]; else g[i] = *sp;
+            row += drow;
+            x += dx;
+            if (x >= w) { x -= w; ++row; }
         }
     }
+}
+
+// Zeroes the margins of nrows canvas rows and the all-zero row kept at index zrow.
+template <int N>
+__device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int w, int padL, int zrow,
+                                                    int tid)
+{
+    constexpr int LDR = Canvas<N>::LDR;
+    for (int row = tid; row < nrows; row += 256) {
+        float *sp = smem + row * LDR;
+        for (int c = 0; c < padL; ++c) sp[c] = 0.0f;
+        for (int c = padL + w; c < N; ++c) sp[c] = 0.0f;
+    }
+    if (tid < N) smem[zrow * LDR + tid] = 0.0f;
 }
 
 // ---------------------------------------------------------------------------------
@@ -106,10 +143,10 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(const floa
     constexpr int T = S::T;
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x;
-    const long x0 = (long)blockIdx.x * T;
+    const long x0 = plane_group<N>(blockIdx.x) * T;
+    if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
-    const int hwp = hw | 1;                           // odd plane stride in the staging area
     const int y_lo = padU & ~1;                       // first canvas row that can be non-zero (even)
     const int y_hi = (padU + h + 1) & ~1;             // one past the last, rounded up to even
 
@@ -124,22 +161,26 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(const floa
     const bool vb = (ib >= 0) && (ib < h);
     const bool row_active = (t < np) && (va || vb);
 
-    // ---- stage the contiguous chunk of planes, TP planes per round ----
+    // ---- stage the contiguous chunk of planes as zero-padded canvas rows, TP planes per round ----
+    constexpr int LDR = Canvas<N>::LDR;
+    const int zrow = S::TP * h;  // an all-zero row for canvas rows outside the plane
     static_for<S::PH>([&](auto hh) {
         constexpr int hs = decltype(hh)::value;
         int nph = np - hs * S::TP;
         nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
         if (hs > 0) __syncthreads();  // previous round fully read
-        copy_planes<true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph, hw, hwp, vec4, tid);
+        zero_canvas_margins<N>(smem, nph * h, w, padL, zrow, tid);
+        copy_canvas<N, true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
         __syncthreads();
         if (row_active && (t / S::TP) == hs) {
-            const float *pa = smem + (t - hs * S::TP) * hwp + ia * w - padL;
-            const float *pb = smem + (t - hs * S::TP) * hwp + ib * w - padL;
-            static_for<N>([&](auto cc) {
-                constexpr int c = decltype(cc)::value;
-                const bool vc = (c >= padL) && (c < padL + w);
-                re[c] = (va && vc) ? pa[c] : 0.0f;
-                im[c] = (vb && vc) ? pb[c] : 0.0f;
+            const int tl = t - hs * S::TP;
+            const float4 *pa = reinterpret_cast<const float4 *>(smem + (va ? tl * h + ia : zrow) * LDR);
+            const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? tl * h + ib : zrow) * LDR);
+            static_for<N / 4>([&](auto jj) {
+                constexpr int j = decltype(jj)::value;
+                const float4 a = pa[j], b = pb[j];
+                re[4 * j] = a.x; re[4 * j + 1] = a.y; re[4 * j + 2] = a.z; re[4 * j + 3] = a.w;
+                im[4 * j] = b.x; im[4 * j + 1] = b.y; im[4 * j + 2] = b.z; im[4 * j + 3] = b.w;
             });
         }
     });
@@ -242,10 +283,10 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void irfft2d_kernel(const flo
     constexpr int T = S::T;
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x;
-    const long x0 = (long)blockIdx.x * T;
+    const long x0 = plane_group<N>(blockIdx.x) * T;
+    if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
-    const int hwp = hw | 1;                           // odd plane stride in the staging area
     const int y_lo = padU & ~1;                       // canvas rows the crop needs
     const int y_hi = (padU + h + 1) & ~1;
 
@@ -323,24 +364,34 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void irfft2d_kernel(const flo
         fft_inplace<N, true>(zr, zi);
         if (bias != nullptr) bv = bias[(x0 + t) % bias_period];
     }
-    // ---- crop (+bias) into the staging area and coalesced copy-out, TP planes per round ----
+    // ---- canvas rows (+bias) into the staging area, cropped coalesced copy-out, TP planes per round ----
+    constexpr int LDR = Canvas<N>::LDR;
     static_for<S::PH>([&](auto hh) {
         constexpr int hs = decltype(hh)::value;
         int nph = np - hs * S::TP;
         nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
         if (hs > 0) __syncthreads();  // previous round copied out
         if (row_active && (t / S::TP) == hs) {
-            float *pa = smem + (t - hs * S::TP) * hwp + ia * w - padL;
-            float *pb = smem + (t - hs * S::TP) * hwp + ib * w - padL;
-            static_for<N>([&](auto cc) {
-                constexpr int c = decltype(cc)::value;
-                const bool vc = (c >= padL) && (c < padL + w);
-                if (va && vc) pa[c] = zr[brev<N>(c)] + bv;
-                if (vb && vc) pb[c] = zi[brev<N>(c)] + bv;
-            });
+            const int tl = t - hs * S::TP;
+            if (va) {
+                float4 *pa = reinterpret_cast<float4 *>(smem + (tl * h + ia) * LDR);
+                static_for<N / 4>([&](auto jj) {
+                    constexpr int j = decltype(jj)::value;
+                    pa[j] = make_float4(zr[brev<N>(4 * j)] + bv, zr[brev<N>(4 * j + 1)] + bv,
+                                        zr[brev<N>(4 * j + 2)] + bv, zr[brev<N>(4 * j + 3)] + bv);
+                });
+            }
+            if (vb) {
+                float4 *pb = reinterpret_cast<float4 *>(smem + (tl * h + ib) * LDR);
+                static_for<N / 4>([&](auto jj) {
+                    constexpr int j = decltype(jj)::value;
+                    pb[j] = make_float4(zi[brev<N>(4 * j)] + bv, zi[brev<N>(4 * j + 1)] + bv,
+                                        zi[brev<N>(4 * j + 2)] + bv, zi[brev<N>(4 * j + 3)] + bv);
+                });
+            }
         }
         __syncthreads();
-        copy_planes<false>(smem, out + (x0 + hs * S::TP) * hw, nph, hw, hwp, vec4, tid);
+        copy_canvas<N, false>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
     });
 }
 
@@ -354,8 +405,8 @@ static size_t fft_lds_bytes(int h, int w, int padU, bool inverse)
     const int y_lo = padU & ~1, y_hi = (padU + h + 1) & ~1;
     const size_t tile = (size_t)(y_hi - y_lo) * S::ROWSTRIDE * sizeof(float2);
     (void)inverse;
-    const size_t plane = (size_t)((h * w) | 1);
-    const size_t stage = (size_t)S::TP * plane * sizeof(float);
+    (void)w;
+    const size_t stage = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
     return ((tile > stage ? tile : stage) + 15) & ~(size_t)15;
 }
 
@@ -372,7 +423,8 @@ static hipError_t launch_fwd(const float *in, float *out, long planes, int h, in
         attr_done = true;
     }
     const size_t lds = fft_lds_bytes<N>(h, w, padU, false);
-    const long blocks = (planes + S::T - 1) / S::T;
+    long blocks = (planes + S::T - 1) / S::T;
+    if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
     const int vec4 = ((reinterpret_cast<uintptr_t>(in) & 15) == 0) && (((long)S::T * h * w) % 4 == 0);
     hipLaunchKernelGGL(rfft2d_kernel<N>, dim3((unsigned)blocks), dim3(256), lds, s, in,
                        reinterpret_cast<float2 *>(out), planes, h, w, padU, padL, vec4);
@@ -392,7 +444,8 @@ static hipError_t launch_inv(const float *in, float *out, long planes, int h, in
         attr_done = true;
     }
     const size_t lds = fft_lds_bytes<N>(h, w, padU, true);
-    const long blocks = (planes + S::T - 1) / S::T;
+    long blocks = (planes + S::T - 1) / S::T;
+    if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
     const int vec4 = ((reinterpret_cast<uintptr_t>(out) & 15) == 0) && (((long)S::T * h * w) % 4 == 0);
     hipLaunchKernelGGL(irfft2d_kernel<N>, dim3((unsigned)blocks), dim3(256), lds, s,
                        reinterpret_cast<const float2 *>(in), out, planes, h, w, padU, padL, bias,
