@@ -192,7 +192,9 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(const floa
     float ar[NLATE > 0 ? NLATE : 1], ai[NLATE > 0 ? NLATE : 1], br[NLATE > 0 ? NLATE : 1], bi[NLATE > 0 ? NLATE : 1];
     float2 *R = reinterpret_cast<float2 *>(smem);
     const int kx = tid / T;  // column pass: lane (t, kx) owns tile column kx of plane t
+    const int nrows = y_hi - y_lo;  // tile rows; row index nrows is an all-zero row
     __syncthreads();  // staging area fully consumed; the tile may overwrite it
+    if (tid < S::KXP * T) R[nrows * S::ROWSTRIDE + tid] = make_float2(0.0f, 0.0f);
     if (row_active) {
         fft_inplace<N, false>(re, im);
         float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
@@ -234,11 +236,12 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(const floa
         __syncthreads();
         if ((t < np) && (kx / S::KXP) == ph) {
             const int kl = kx - ph * S::KXP;
+            const float2 *col = R + kl * T + t;
             static_for<N>([&](auto yy) {
                 constexpr int y = decltype(yy)::value;
-                const bool vy = (y >= y_lo) && (y < y_hi);
-                float2 v = make_float2(0.0f, 0.0f);
-                if (vy) v = R[(y - y_lo) * S::ROWSTRIDE + kl * T + t];
+                // canvas rows outside the plane read the zero row (uniform select, no branch)
+                const int row = ((y >= y_lo) && (y < y_hi)) ? (y - y_lo) : nrows;
+                const float2 v = col[row * S::ROWSTRIDE];
                 re[y] = v.x;
                 im[y] = v.y;
             });
@@ -248,11 +251,16 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(const floa
     // ---- column FFT and frequency-major store, all lanes at once ----
     if (t < np) {
         fft_inplace<N, false>(re, im);
-        float2 *o = out + x0 + t;
+        // address = uniform base (frequency row ky, first plane of the group) + 32-bit lane offset
+        const unsigned voff = (unsigned)(((long)kx * planes + t) * (long)sizeof(float2));
+        const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + t) * (long)sizeof(float2));
+        char *obase = reinterpret_cast<char *>(out + x0);
+        const long rowbytes = (long)S::NH * planes * (long)sizeof(float2);
         if (kx != 0) {
             static_for<N>([&](auto kk) {
                 constexpr int ky = decltype(kk)::value;
-                o[(long)(ky * S::NH + kx) * planes] = make_float2(re[brev<N>(ky)], im[brev<N>(ky)]);
+                *reinterpret_cast<float2 *>(obase + ky * rowbytes + voff) =
+                    make_float2(re[brev<N>(ky)], im[brev<N>(ky)]);
             });
         } else {
             // C = FFT(col0 + i colNyq), both real sequences: untangle
@@ -261,8 +269,10 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(const floa
                 constexpr int kn = (N - ky) % N;
                 const float zr = re[brev<N>(ky)], zi = im[brev<N>(ky)];
                 const float nr = re[brev<N>(kn)], ni = im[brev<N>(kn)];
-                o[(long)(ky * S::NH + 0) * planes] = make_float2(0.5f * (zr + nr), 0.5f * (zi - ni));
-                o[(long)(ky * S::NH + N / 2) * planes] = make_float2(0.5f * (zi + ni), 0.5f * (nr - zr));
+                *reinterpret_cast<float2 *>(obase + ky * rowbytes + voff) =
+                    make_float2(0.5f * (zr + nr), 0.5f * (zi - ni));
+                *reinterpret_cast<float2 *>(obase + ky * rowbytes + vnyq) =
+                    make_float2(0.5f * (zi + ni), 0.5f * (nr - zr));
             });
         }
     }
@@ -297,11 +307,15 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void irfft2d_kernel(const flo
     // ---- column pass: lane (t, kx) fetches its whole column and transforms it, all lanes at once ----
     const int kx = tid / T;
     if (t < np) {
-        const float2 *src = in + x0 + t;
+        // address = uniform base (frequency row ky, first plane of the group) + 32-bit lane offset
+        const unsigned voff = (unsigned)(((long)kx * planes + t) * (long)sizeof(float2));
+        const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + t) * (long)sizeof(float2));
+        const char *ibase = reinterpret_cast<const char *>(in + x0);
+        const long rowbytes = (long)S::NH * planes * (long)sizeof(float2);
         if (kx != 0) {
             static_for<N>([&](auto kk) {
                 constexpr int ky = decltype(kk)::value;
-                const float2 v = src[(long)(ky * S::NH + kx) * planes];
+                const float2 v = *reinterpret_cast<const float2 *>(ibase + ky * rowbytes + voff);
                 re[ky] = v.x;
                 im[ky] = v.y;
             });
@@ -309,8 +323,8 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void irfft2d_kernel(const flo
             // pack columns 0 and N/2 (each the spectrum of a real sequence): C = X0 + i XN
             static_for<N>([&](auto kk) {
                 constexpr int ky = decltype(kk)::value;
-                const float2 a = src[(long)(ky * S::NH + 0) * planes];
-                const float2 b = src[(long)(ky * S::NH + N / 2) * planes];
+                const float2 a = *reinterpret_cast<const float2 *>(ibase + ky * rowbytes + voff);
+                const float2 b = *reinterpret_cast<const float2 *>(ibase + ky * rowbytes + vnyq);
                 re[ky] = a.x - b.y;
                 im[ky] = a.y + b.x;
             });
@@ -327,16 +341,19 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void irfft2d_kernel(const flo
     const bool row_active = (t < np) && (va || vb);
     // Z[k] = Ya[k] + i Yb[k], k = 0..N-1, with Y[N-k] = conj Y[k]
     float zr[N], zi[N];
+    const int nrows = y_hi - y_lo;  // tile rows; row index nrows is a dummy row
 
     static_for<S::PH>([&](auto pp) {
         constexpr int ph = decltype(pp)::value;
         if (ph > 0) __syncthreads();  // previous phase's tile fully read
         if ((t < np) && (kx / S::KXP) == ph) {
             const int kl = kx - ph * S::KXP;
+            float2 *col = R + kl * T + t;
             static_for<N>([&](auto yy) {
                 constexpr int y = decltype(yy)::value;
-                if ((y >= y_lo) && (y < y_hi))
-                    R[(y - y_lo) * S::ROWSTRIDE + kl * T + t] = make_float2(re[brev<N>(y)], im[brev<N>(y)]);
+                // rows the crop does not need land in a dummy row (uniform select, no branch)
+                const int row = ((y >= y_lo) && (y < y_hi)) ? (y - y_lo) : nrows;
+                col[row * S::ROWSTRIDE] = make_float2(re[brev<N>(y)], im[brev<N>(y)]);
             });
         }
         __syncthreads();
@@ -403,7 +420,7 @@ static size_t fft_lds_bytes(int h, int w, int padU, bool inverse)
 {
     using S = FftShape<N>;
     const int y_lo = padU & ~1, y_hi = (padU + h + 1) & ~1;
-    const size_t tile = (size_t)(y_hi - y_lo) * S::ROWSTRIDE * sizeof(float2);
+    const size_t tile = (size_t)(y_hi - y_lo + 1) * S::ROWSTRIDE * sizeof(float2);
     (void)inverse;
     (void)w;
     const size_t stage = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
@@ -453,9 +470,13 @@ static hipError_t launch_inv(const float *in, float *out, long planes, int h, in
     return hipGetLastError();
 }
 
+// the kernels address a frequency row with 32-bit lane offsets
+static bool planes_ok(int N, long planes) { return planes > 0 && (long)(N / 2 + 1) * planes * 8 < (1L << 31); }
+
 hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                          int padL, hipStream_t s)
 {
+    if (!planes_ok(N, planes)) return hipErrorInvalidValue;
     switch (N) {
         case 8: return launch_fwd<8>(in, out, planes, h, w, padU, padL, s);
         case 16: return launch_fwd<16>(in, out, planes, h, w, padU, padL, s);
@@ -468,6 +489,7 @@ hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h,
 hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                           int padL, const float *bias, int bias_period, hipStream_t s)
 {
+    if (!planes_ok(N, planes)) return hipErrorInvalidValue;
     switch (N) {
         case 8: return launch_inv<8>(in, out, planes, h, w, padU, padL, bias, bias_period, s);
         case 16: return launch_inv<16>(in, out, planes, h, w, padU, padL, bias, bias_period, s);
