@@ -113,6 +113,8 @@ struct StageTimer {
             (void)hipEventRecord(p->ev[0], s);
         }
     }
+    // number of back-to-back launches of each stage (1 unless the plan is timed)
+    int reps() const { return p->timed > 0 ? p->timed : 1; }
     void done(int stage)
     {
         if (!p->timed) return;
@@ -129,7 +131,7 @@ struct StageTimer {
             float ms = 0.0f;
             e = hipEventElapsedTime(&ms, p->ev[i], p->ev[i + 1]);
             if (e != hipSuccess) return fail_hip(e, "hipEventElapsedTime");
-            p->stage_ms[slot[i]] = ms;
+            p->stage_ms[slot[i]] = ms / (float)reps();
         }
         return FBFC_OK;
     }
@@ -139,6 +141,16 @@ struct StageTimer {
     do {                                                       \
         hipError_t e_ = (expr);                                \
         if (e_ != hipSuccess) return fail_hip(e_, what);       \
+    } while (0)
+
+// A stage of a pass: launched once, or tm.reps() times back to back when the plan is timed
+// (every stage is a pure function of its inputs, so repeating it changes no result).
+#define FBFC_STAGE(tm, expr, what)                             \
+    do {                                                       \
+        for (int r_ = 0; r_ < (tm).reps(); ++r_) {             \
+            hipError_t e_ = (expr);                            \
+            if (e_ != hipSuccess) return fail_hip(e_, what);   \
+        }                                                      \
     } while (0)
 
 }  // namespace
@@ -233,7 +245,7 @@ int fbfc_plan_set_timed(fbfc_plan *p, int on)
         for (hipEvent_t &ev : p->ev) FBFC_TRY(hipEventCreate(&ev), "hipEventCreate");
         p->ev_made = true;
     }
-    p->timed = on ? 1 : 0;
+    p->timed = on > 0 ? on : 0;
     return FBFC_OK;
 }
 
@@ -253,21 +265,21 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     const fbfc_conv_desc &d = p->d;
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
-    FBFC_TRY(fbfc::launch_rfft2d(N, input, p->in_freq, (long)d.batch * d.in_planes, d.in_h, d.in_w,
+    FBFC_STAGE(tm, fbfc::launch_rfft2d(N, input, p->in_freq, (long)d.batch * d.in_planes, d.in_h, d.in_w,
                                  d.pad_h, d.pad_w, s), "rfft2d(input)");
     p->have_in = true;
     tm.done(FBFC_STAGE_FFT_A);
-    FBFC_TRY(fbfc::launch_rfft2d(N, weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w,
+    FBFC_STAGE(tm, fbfc::launch_rfft2d(N, weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w,
                                  0, 0, s), "rfft2d(weight)");
     p->have_w = true;
     tm.done(FBFC_STAGE_FFT_B);
     float *res = p->reuse ? p->res_freq : p->out_freq;
     if (!p->reuse) p->have_out = false;
     // O[b][f] = 1/N^2 sum_p I[b][p] conj(W[f][p])   (SpatialConvolutionFBFFT.lua:157-164)
-    FBFC_TRY(fbfc::launch_cgemm_freq(0, p->in_freq, p->w_freq, res, Q, d.batch, d.out_planes,
+    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(0, p->in_freq, p->w_freq, res, Q, d.batch, d.out_planes,
                                      d.in_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(fprop)");
     tm.done(FBFC_STAGE_MM);
-    FBFC_TRY(fbfc::launch_irfft2d(N, res, output, (long)d.batch * d.out_planes, p->info.out_h,
+    FBFC_STAGE(tm, fbfc::launch_irfft2d(N, res, output, (long)d.batch * d.out_planes, p->info.out_h,
                                   p->info.out_w, 0, 0, bias, d.out_planes, s), "irfft2d(output)");
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();
@@ -282,12 +294,12 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     const fbfc_conv_desc &d = p->d;
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
-    FBFC_TRY(fbfc::launch_rfft2d(N, grad_output, p->out_freq, (long)d.batch * d.out_planes,
+    FBFC_STAGE(tm, fbfc::launch_rfft2d(N, grad_output, p->out_freq, (long)d.batch * d.out_planes,
                                  p->info.out_h, p->info.out_w, 0, 0, s), "rfft2d(gradOutput)");
     p->have_out = true;
     tm.done(FBFC_STAGE_FFT_A);
     if (!((p->reuse & FBFC_REUSE_WEIGHT) && p->have_w)) {
-        FBFC_TRY(fbfc::launch_rfft2d(N, weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h,
+        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h,
                                      d.k_w, 0, 0, s), "rfft2d(weight)");
         p->have_w = true;
         tm.done(FBFC_STAGE_FFT_B);
@@ -295,10 +307,10 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     float *res = p->reuse ? p->res_freq : p->in_freq;
     if (!p->reuse) p->have_in = false;
     // GI[b][p] = 1/N^2 sum_f GO[b][f] W[f][p]   (SpatialConvolutionFBFFT.lua:244-251)
-    FBFC_TRY(fbfc::launch_cgemm_freq(1, p->out_freq, p->w_freq, res, Q, d.batch, d.in_planes,
+    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(1, p->out_freq, p->w_freq, res, Q, d.batch, d.in_planes,
                                      d.out_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(bprop)");
     tm.done(FBFC_STAGE_MM);
-    FBFC_TRY(fbfc::launch_irfft2d(N, res, grad_input, (long)d.batch * d.in_planes, d.in_h, d.in_w,
+    FBFC_STAGE(tm, fbfc::launch_irfft2d(N, res, grad_input, (long)d.batch * d.in_planes, d.in_h, d.in_w,
                                   d.pad_h, d.pad_w, nullptr, 1, s), "irfft2d(gradInput)");
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();
@@ -314,18 +326,18 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
     if (grad_bias != nullptr) {
-        FBFC_TRY(fbfc::launch_bias_grad(grad_output, grad_bias, scale, d.batch, d.out_planes,
+        FBFC_STAGE(tm, fbfc::launch_bias_grad(grad_output, grad_bias, scale, d.batch, d.out_planes,
                                         p->info.out_h * p->info.out_w, p->scratch, s), "bias grad");
         tm.done(FBFC_STAGE_BIAS_GRAD);
     }
     if (!((p->reuse & FBFC_REUSE_OUTPUT) && p->have_out)) {
-        FBFC_TRY(fbfc::launch_rfft2d(N, grad_output, p->out_freq, (long)d.batch * d.out_planes,
+        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, grad_output, p->out_freq, (long)d.batch * d.out_planes,
                                      p->info.out_h, p->info.out_w, 0, 0, s), "rfft2d(gradOutput)");
         p->have_out = true;
         tm.done(FBFC_STAGE_FFT_A);
     }
     if (!((p->reuse & FBFC_REUSE_INPUT) && p->have_in)) {
-        FBFC_TRY(fbfc::launch_rfft2d(N, input, p->in_freq, (long)d.batch * d.in_planes, d.in_h,
+        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, input, p->in_freq, (long)d.batch * d.in_planes, d.in_h,
                                      d.in_w, d.pad_h, d.pad_w, s), "rfft2d(input)");
         p->have_in = true;
         tm.done(FBFC_STAGE_FFT_B);
@@ -333,10 +345,10 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     float *res = p->reuse ? p->res_freq : p->w_freq;
     if (!p->reuse) p->have_w = false;
     // GW[f][p] = scale/N^2 sum_b conj(GO[b][f]) I[b][p]   (SpatialConvolutionFBFFT.lua:337-344)
-    FBFC_TRY(fbfc::launch_cgemm_freq(2, p->out_freq, p->in_freq, res, Q, d.out_planes, d.in_planes,
+    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(2, p->out_freq, p->in_freq, res, Q, d.out_planes, d.in_planes,
                                      d.batch, scale / ((float)N * (float)N), 0, s), "cgemm(accGrad)");
     tm.done(FBFC_STAGE_MM);
-    FBFC_TRY(fbfc::launch_irfft2d(N, res, grad_weight, (long)d.out_planes * d.in_planes, d.k_h, d.k_w,
+    FBFC_STAGE(tm, fbfc::launch_irfft2d(N, res, grad_weight, (long)d.out_planes * d.in_planes, d.k_h, d.k_w,
                                   0, 0, nullptr, 1, s), "irfft2d(gradWeight)");
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();

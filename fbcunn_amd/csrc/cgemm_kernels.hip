@@ -200,6 +200,154 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Split-K kernel for small problems (few 64x64 tiles per CU).
+//
+// With only a handful of output tiles per SIMD, whole tiles cannot be balanced over the 1024
+// SIMDs (config 4 has 2.25 32x32-complex blocks per SIMD).  Here a workgroup owns ONE 32x32
+// complex block and its four waves each contract a quarter of K, so the unit of scheduling
+// is a quarter block (9 per SIMD for config 4).  Operands go straight from global memory into
+// the MFMA operand registers (each lane loads exactly the k' it feeds: 64 contiguous bytes of
+// a K-contiguous row, or one complex per row of a row-contiguous operand); LDS is used only
+// to add the four partial accumulators.  Preconditions: M % 32 == N % 32 == 0, K % 64 == 0.
+// ---------------------------------------------------------------------------------------
+template <int MODE>
+__device__ __forceinline__ void splitk_load(const float2 *__restrict__ Aq, const float2 *__restrict__ Bq,
+                                            int M, int N, int K, int arow, int bcol, int k0, int h,
+                                            float (&a)[16], float (&b)[16])
+{
+    constexpr bool A_KC = (MODE != 2);
+    constexpr bool B_KC = (MODE == 0);
+    if (A_KC) {  // A[m][k]: 8 consecutive complex of row arow
+        const float4 *p = reinterpret_cast<const float4 *>(Aq + (long)arow * K + k0 + 8 * h);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4 v = p[j];
+            a[4 * j] = v.x; a[4 * j + 1] = v.y; a[4 * j + 2] = v.z; a[4 * j + 3] = v.w;
+        }
+    } else {     // A[k][m]: column arow of 8 consecutive rows
+        const float2 *p = Aq + (long)(k0 + 8 * h) * M + arow;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float2 v = p[(long)j * M];
+            a[2 * j] = v.x; a[2 * j + 1] = v.y;
+        }
+    }
+    if (B_KC) {  // B[n][k]
+        const float4 *p = reinterpret_cast<const float4 *>(Bq + (long)bcol * K + k0 + 8 * h);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4 v = p[j];
+            b[4 * j] = v.x; b[4 * j + 1] = v.y; b[4 * j + 2] = v.z; b[4 * j + 3] = v.w;
+        }
+    } else {     // B[k][n]
+        const float2 *p = Bq + (long)(k0 + 8 * h) * N + bcol;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float2 v = p[(long)j * N];
+            b[2 * j] = v.x; b[2 * j + 1] = v.y;
+        }
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ void splitk_mfma(const float (&a)[16], const float (&b)[16], floatx16 &cre,
+                                            floatx16 &cim)
+{
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float ar = a[2 * j], ai = a[2 * j + 1], br = b[2 * j], bi = b[2 * j + 1];
+        if (MODE == 0) {         // A conj(B)
+            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, cre, 0, 0, 0);
+            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, -bi, cim, 0, 0, 0);
+            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, bi, cre, 0, 0, 0);
+            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, br, cim, 0, 0, 0);
+        } else if (MODE == 1) {  // A B
+            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, cre, 0, 0, 0);
+            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, bi, cim, 0, 0, 0);
+            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, -bi, cre, 0, 0, 0);
+            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, br, cim, 0, 0, 0);
+        } else {                 // conj(A)^T B
+            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, cre, 0, 0, 0);
+            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, bi, cim, 0, 0, 0);
+            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, bi, cre, 0, 0, 0);
+            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, -br, cim, 0, 0, 0);
+        }
+    }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restrict__ A,
+                                                           const float2 *__restrict__ B,
+                                                           float2 *__restrict__ C, int M, int N, int K,
+                                                           float alpha, int accumulate, int tilesM,
+                                                           int tilesN, int total_wgs, int chunk)
+{
+    __shared__ float red[4][32][64];  // [wave][accumulator register][lane]
+
+    const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
+    if (wg >= total_wgs) return;
+    const int tiles = tilesM * tilesN;
+    const int q = wg / tiles;
+    const int tile = wg - q * tiles;
+    const int m0 = (tile / tilesN) * 32;
+    const int n0 = (tile % tilesN) * 32;
+    const float2 *Aq = A + (long)q * M * K;
+    const float2 *Bq = B + (long)q * N * K;
+    float2 *Cq = C + (long)q * M * N;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int li = lane & 31, h = lane >> 5;
+    const int kq = K >> 2;                      // this wave's share of K (a multiple of 16)
+    const int kbeg = wave * kq, nkt = kq >> 4;  // K-tiles of 16 complex
+
+    floatx16 cre, cim;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { cre[r] = 0.f; cim[r] = 0.f; }
+
+    float a0[16], b0[16], a1[16], b1[16];
+    splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg, h, a0, b0);
+    int kt = 0;
+    for (; kt + 1 < nkt; kt += 2) {
+        splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * (kt + 1), h, a1, b1);
+        __builtin_amdgcn_sched_barrier(0);
+        splitk_mfma<MODE>(a0, b0, cre, cim);
+        __builtin_amdgcn_sched_barrier(0);
+        // the last prefetch of an even count re-reads the final tile and is not used
+        const int knext = (kt + 2 < nkt) ? kt + 2 : kt + 1;
+        splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * knext, h, a0, b0);
+        __builtin_amdgcn_sched_barrier(0);
+        splitk_mfma<MODE>(a1, b1, cre, cim);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kt < nkt) splitk_mfma<MODE>(a0, b0, cre, cim);
+
+    // add the four partial accumulators: every wave finalises 8 rows of the block
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        red[wave][r][lane] = cre[r];
+        red[wave][16 + r][lane] = cim[r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+        const int r = 4 * wave + rr;
+        const float sre = (red[0][r][lane] + red[1][r][lane]) + (red[2][r][lane] + red[3][r][lane]);
+        const float sim = (red[0][16 + r][lane] + red[1][16 + r][lane]) +
+                          (red[2][16 + r][lane] + red[3][16 + r][lane]);
+        // accumulator register r of lane (li, h) is C[8*(r/4) + 4*h + r%4][li] of the block
+        const int row = m0 + 8 * wave + 4 * h + rr;
+        float2 v = make_float2(alpha * sre, alpha * sim);
+        float2 *dst = Cq + (long)row * N + n0 + li;
+        if (accumulate) {
+            const float2 o = *dst;
+            v.x += o.x;
+            v.y += o.y;
+        }
+        *dst = v;
+    }
+}
+
 template <int MODE>
 static hipError_t launch_mode(const float *A, const float *B, float *C, int n_freq, int m, int n,
                               int k, float alpha, int accumulate, hipStream_t s)
@@ -207,6 +355,18 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
     const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
     const long total = (long)n_freq * tilesM * tilesN;
     if (total <= 0 || total > 0x7fffff00L) return hipErrorInvalidValue;
+    // fewer than 8 tiles of 64x64 per CU: schedule quarter blocks instead (see cgemm_splitk_kernel)
+    const bool aligned16 = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
+    if (total < 8 * 256 && (m % 32) == 0 && (n % 32) == 0 && (k % 64) == 0 && aligned16) {
+        const int tm = m / 32, tn = n / 32;
+        const long tot32 = (long)n_freq * tm * tn;
+        const int chunk = (int)((tot32 + 7) / 8);
+        hipLaunchKernelGGL(cgemm_splitk_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
+                           reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
+                           reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tm, tn,
+                           (int)tot32, chunk);
+        return hipGetLastError();
+    }
     const int chunk = (int)((total + 7) / 8);
     hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),

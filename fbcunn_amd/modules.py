@@ -135,7 +135,7 @@ class SpatialConvolutionFFT:
             if self._reuse_bits:
                 check(lib().fbfc_plan_set_reuse(plan.handle, self._reuse_bits))
             self._plans[key] = plan
-        check(lib().fbfc_plan_set_timed(plan.handle, 1 if self.timed else 0))
+        check(lib().fbfc_plan_set_timed(plan.handle, int(self.timed)))  # reps per stage, 0 = off
         return plan
 
     def _check_input(self, input):
@@ -144,7 +144,7 @@ class SpatialConvolutionFFT:
             raise ValueError("input has %d planes, module expects %d" % (input.size(1), self.nInputPlane))
 
     def stageTimes(self, input):
-        """ms per stage of the last pass run with self.timed = True (dict)."""
+        """Mean ms per launch of each stage of the last pass run with self.timed = reps > 0 (dict)."""
         plan = self._plan_for(input.size(0), input.size(2), input.size(3))
         ms = (ctypes.c_float * len(_lib.STAGE_NAMES))()
         check(lib().fbfc_plan_stage_ms(plan.handle, ms, len(_lib.STAGE_NAMES)))

@@ -27,6 +27,8 @@ def _c(a):
 SHAPES = [  # Q, m, n, k
     (5, 64, 64, 16), (3, 128, 64, 64), (4, 32, 32, 32), (7, 1, 1, 1), (6, 3, 5, 7),
     (2, 65, 33, 17), (3, 70, 130, 40), (2, 64, 256, 96), (9, 16, 16, 4), (2, 100, 20, 129),
+    # small aligned problems take the split-K kernel (M, N multiples of 32, K of 64)
+    (4, 32, 32, 64), (2, 96, 160, 128), (3, 128, 128, 128), (5, 64, 32, 192), (144, 128, 128, 128),
 ]
 
 
@@ -50,8 +52,8 @@ def test_transpose_mm(nn, mode, Q, m, n, k):
     assert np.abs(got - want).max() <= TOL * np.abs(want).max()
 
 
-def test_accumulate_flag(nn):
-    Q, m, n, k = 3, 40, 50, 20
+@pytest.mark.parametrize("Q,m,n,k", [(3, 40, 50, 20), (3, 64, 96, 64)])
+def test_accumulate_flag(nn, Q, m, n, k):
     A, B = synth.uniform(3, (Q, m, k, 2)), synth.uniform(4, (Q, k, n, 2))
     C0 = synth.uniform(5, (Q, m, n, 2))
     C = dev(C0)
