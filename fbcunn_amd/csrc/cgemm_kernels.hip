@@ -20,6 +20,8 @@
 // register-prefetch double buffering through LDS.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "kernels.h"
 
 namespace fbfc {
@@ -276,76 +278,132 @@ __device__ __forceinline__ void splitk_mfma(const float (&a)[16], const float (&
     }
 }
 
-template <int MODE>
+template <int MODE, int SK>
 __global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restrict__ A,
                                                            const float2 *__restrict__ B,
                                                            float2 *__restrict__ C, int M, int N, int K,
                                                            float alpha, int accumulate, int tilesM,
-                                                           int tilesN, int total_wgs, int chunk)
+                                                           int tilesN, int total_tiles, int total_wgs,
+                                                           int chunk)
 {
-    __shared__ float red[4][32][64];  // [wave][accumulator register][lane]
+    constexpr int TPW = 4 / SK;  // 32x32 blocks per workgroup; SK waves share one block's K range
+    __shared__ float red[SK > 1 ? 4 : 1][32][64];  // [wave][accumulator register][lane]
 
     const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
     if (wg >= total_wgs) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int li = lane & 31, h = lane >> 5;
+    const int ks = wave % SK;  // which share of K
+    const int gtile = wg * TPW + wave / SK;
+    // consecutive blocks run along N: the waves of a workgroup share rows of A (through L1)
+    const bool live = gtile < total_tiles;
     const int tiles = tilesM * tilesN;
-    const int q = wg / tiles;
-    const int tile = wg - q * tiles;
+    const int q = live ? gtile / tiles : 0;
+    const int tile = live ? gtile - q * tiles : 0;
     const int m0 = (tile / tilesN) * 32;
     const int n0 = (tile % tilesN) * 32;
     const float2 *Aq = A + (long)q * M * K;
     const float2 *Bq = B + (long)q * N * K;
     float2 *Cq = C + (long)q * M * N;
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int li = lane & 31, h = lane >> 5;
-    const int kq = K >> 2;                      // this wave's share of K (a multiple of 16)
-    const int kbeg = wave * kq, nkt = kq >> 4;  // K-tiles of 16 complex
+    const int kq = K / SK;                    // this wave's share of K (a multiple of 16)
+    const int kbeg = ks * kq, nkt = kq >> 4;  // K-tiles of 16 complex
 
     floatx16 cre, cim;
 #pragma unroll
     for (int r = 0; r < 16; ++r) { cre[r] = 0.f; cim[r] = 0.f; }
 
-    float a0[16], b0[16], a1[16], b1[16];
-    splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg, h, a0, b0);
-    int kt = 0;
-    for (; kt + 1 < nkt; kt += 2) {
-        splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * (kt + 1), h, a1, b1);
-        __builtin_amdgcn_sched_barrier(0);
-        splitk_mfma<MODE>(a0, b0, cre, cim);
-        __builtin_amdgcn_sched_barrier(0);
-        // the last prefetch of an even count re-reads the final tile and is not used
-        const int knext = (kt + 2 < nkt) ? kt + 2 : kt + 1;
-        splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * knext, h, a0, b0);
-        __builtin_amdgcn_sched_barrier(0);
-        splitk_mfma<MODE>(a1, b1, cre, cim);
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    if (kt < nkt) splitk_mfma<MODE>(a0, b0, cre, cim);
-
-    // add the four partial accumulators: every wave finalises 8 rows of the block
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        red[wave][r][lane] = cre[r];
-        red[wave][16 + r][lane] = cim[r];
-    }
-    __syncthreads();
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr) {
-        const int r = 4 * wave + rr;
-        const float sre = (red[0][r][lane] + red[1][r][lane]) + (red[2][r][lane] + red[3][r][lane]);
-        const float sim = (red[0][16 + r][lane] + red[1][16 + r][lane]) +
-                          (red[2][16 + r][lane] + red[3][16 + r][lane]);
-        // accumulator register r of lane (li, h) is C[8*(r/4) + 4*h + r%4][li] of the block
-        const int row = m0 + 8 * wave + 4 * h + rr;
-        float2 v = make_float2(alpha * sre, alpha * sim);
-        float2 *dst = Cq + (long)row * N + n0 + li;
-        if (accumulate) {
-            const float2 o = *dst;
-            v.x += o.x;
-            v.y += o.y;
+    if (live) {
+        float a0[16], b0[16], a1[16], b1[16];
+        splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg, h, a0, b0);
+        int kt = 0;
+        for (; kt + 1 < nkt; kt += 2) {
+            splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * (kt + 1), h, a1, b1);
+            __builtin_amdgcn_sched_barrier(0);
+            splitk_mfma<MODE>(a0, b0, cre, cim);
+            __builtin_amdgcn_sched_barrier(0);
+            // the last prefetch of an even count re-reads the final tile and is not used
+            const int knext = (kt + 2 < nkt) ? kt + 2 : kt + 1;
+            splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * knext, h, a0, b0);
+            __builtin_amdgcn_sched_barrier(0);
+            splitk_mfma<MODE>(a1, b1, cre, cim);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        *dst = v;
+        if (kt < nkt) splitk_mfma<MODE>(a0, b0, cre, cim);
     }
+
+    if constexpr (SK == 1) {
+        if (!live) return;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            // accumulator register r of lane (li, h) is C[8*(r/4) + 4*h + r%4][li] of the block
+            const int row = m0 + 8 * (r / 4) + 4 * h + (r % 4);
+            float2 v = make_float2(alpha * cre[r], alpha * cim[r]);
+            float2 *dst = Cq + (long)row * N + n0 + li;
+            if (accumulate) {
+                const float2 o = *dst;
+                v.x += o.x;
+                v.y += o.y;
+            }
+            *dst = v;
+        }
+    } else {
+        // add the SK partial accumulators of a block: each of its waves finalises 16/SK registers
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            red[wave][r][lane] = cre[r];
+            red[wave][16 + r][lane] = cim[r];
+        }
+        __syncthreads();
+        if (!live) return;
+        const int w0 = wave - ks;  // first wave of this block
+        constexpr int RPW = 16 / SK;
+#pragma unroll
+        for (int rr = 0; rr < RPW; ++rr) {
+            const int r = RPW * ks + rr;
+            float sre = 0.f, sim = 0.f;
+#pragma unroll
+            for (int v = 0; v < SK; ++v) {
+                sre += red[w0 + v][r][lane];
+                sim += red[w0 + v][16 + r][lane];
+            }
+            const int row = m0 + 8 * (r / 4) + 4 * h + (r % 4);
+            float2 v = make_float2(alpha * sre, alpha * sim);
+            float2 *dst = Cq + (long)row * N + n0 + li;
+            if (accumulate) {
+                const float2 o = *dst;
+                v.x += o.x;
+                v.y += o.y;
+            }
+            *dst = v;
+        }
+    }
+}
+
+template <int MODE, int SK>
+static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_freq, int m, int n,
+                                int k, float alpha, int accumulate, hipStream_t s)
+{
+    const int tm = m / 32, tn = n / 32;
+    const long tot32 = (long)n_freq * tm * tn;
+    const long wgs = (tot32 * SK + 3) / 4;
+    const int chunk = (int)((wgs + 7) / 8);
+    hipLaunchKernelGGL((cgemm_splitk_kernel<MODE, SK>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
+                       reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
+                       reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tm, tn, (int)tot32,
+                       (int)wgs, chunk);
+    return hipGetLastError();
+}
+
+// FBFC_CGEMM_SPLITK = 0 (LDS-tiled kernel), 1, 2 or 4 forces a kernel variant (for measurements).
+static int splitk_override()
+{
+    static int v = -2;
+    if (v == -2) {
+        const char *e = getenv("FBFC_CGEMM_SPLITK");
+        v = (e != nullptr) ? atoi(e) : -1;
+    }
+    return v;
 }
 
 template <int MODE>
@@ -355,17 +413,20 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
     const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
     const long total = (long)n_freq * tilesM * tilesN;
     if (total <= 0 || total > 0x7fffff00L) return hipErrorInvalidValue;
-    // fewer than 8 tiles of 64x64 per CU: schedule quarter blocks instead (see cgemm_splitk_kernel)
+    // Register-fed kernel when the shape allows it (blocks of 32, K-tiles of 16, 16-byte aligned
+    // operands).  The fewer blocks there are per SIMD, the more waves share one block's K range.
     const bool aligned16 = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
-    if (total < 8 * 256 && (m % 32) == 0 && (n % 32) == 0 && (k % 64) == 0 && aligned16) {
-        const int tm = m / 32, tn = n / 32;
-        const long tot32 = (long)n_freq * tm * tn;
-        const int chunk = (int)((tot32 + 7) / 8);
-        hipLaunchKernelGGL(cgemm_splitk_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
-                           reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
-                           reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tm, tn,
-                           (int)tot32, chunk);
-        return hipGetLastError();
+    const long tot32 = (long)n_freq * (m / 32) * (n / 32);
+    if ((m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 && tot32 * 4 < 0x7fffff00L) {
+        const int force = splitk_override();
+        int sk = 0;
+        if (force >= 0) sk = force;
+        else if (tot32 < 4 * 1024 && (k % 64) == 0) sk = 4;
+        else if (tot32 < 8 * 1024 && (k % 32) == 0) sk = 2;
+        else if (MODE != 0) sk = 1;   // K-contiguous operands on both sides do as well through LDS
+        if (sk == 4 && (k % 64) == 0) return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
+        if (sk == 2 && (k % 32) == 0) return launch_splitk<MODE, 2>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
+        if (sk == 1) return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
     }
     const int chunk = (int)((total + 7) / 8);
     hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
