@@ -51,14 +51,15 @@ def stage_model(cfg, pass_, n, q):
         return {"fft_a": ("hbm", fft(B * F, o)), "fft_b": ("hbm", fft(F * P, k)),
                 "mm": ("mfma", mm_flops(B, P, F), mm_bytes(B, P, F)),
                 "ifft": ("hbm", fft(B * P, H))}
-    return {"bias_grad": ("hbm", 4 * B * F * o * o),
+    # the bias gradient is read off the zero-frequency row of FFT(gradOutput): B*F complex numbers
+    return {"bias_grad": ("hbm", 8 * B * F),
             "fft_a": ("hbm", fft(B * F, o)), "fft_b": ("hbm", fft(B * P, H)),
             "mm": ("mfma", mm_flops(F, P, B), mm_bytes(F, P, B)),
             "ifft": ("hbm", fft(F * P, k))}
 
 
 KERNEL_OF_STAGE = {"fft_a": "rfft2d_kernel", "fft_b": "rfft2d_kernel", "mm": "cgemm_freq_kernel",
-                   "ifft": "irfft2d_kernel", "bias_grad": "bias_grad_partial_kernel"}
+                   "ifft": "irfft2d_kernel", "bias_grad": "bias_grad_dc_kernel"}
 
 
 def make_layer(nn, torch, synth, cfg):

@@ -182,7 +182,6 @@ int fbfc_plan_create(const fbfc_conv_desc *desc, fbfc_plan **out)
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->in_freq), info.input_freq_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->w_freq), info.weight_freq_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->out_freq), info.output_freq_bytes);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->scratch), info.scratch_bytes);
     if (e != hipSuccess) {
         const bool oom = (e == hipErrorOutOfMemory);
         (void)hipGetLastError();
@@ -265,14 +264,19 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     const fbfc_conv_desc &d = p->d;
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
-    FBFC_STAGE(tm, fbfc::launch_rfft2d(N, input, p->in_freq, (long)d.batch * d.in_planes, d.in_h, d.in_w,
-                                 d.pad_h, d.pad_w, s), "rfft2d(input)");
+    const fbfc::FwdArgs fin = {input, p->in_freq, (long)d.batch * d.in_planes, d.in_h, d.in_w, d.pad_h, d.pad_w};
+    const fbfc::FwdArgs fw = {weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w, 0, 0};
+    if (!p->timed) {  // both forward FFTs in one launch; timed plans keep them apart to time each
+        FBFC_TRY(fbfc::launch_rfft2d_pair(N, fin, fw, s), "rfft2d(input, weight)");
+    } else {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fin.in, fin.out, fin.planes, fin.h, fin.w, fin.padU, fin.padL, s),
+                   "rfft2d(input)");
+        tm.done(FBFC_STAGE_FFT_A);
+        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fw.in, fw.out, fw.planes, fw.h, fw.w, 0, 0, s), "rfft2d(weight)");
+        tm.done(FBFC_STAGE_FFT_B);
+    }
     p->have_in = true;
-    tm.done(FBFC_STAGE_FFT_A);
-    FBFC_STAGE(tm, fbfc::launch_rfft2d(N, weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w,
-                                 0, 0, s), "rfft2d(weight)");
     p->have_w = true;
-    tm.done(FBFC_STAGE_FFT_B);
     float *res = p->reuse ? p->res_freq : p->out_freq;
     if (!p->reuse) p->have_out = false;
     // O[b][f] = 1/N^2 sum_p I[b][p] conj(W[f][p])   (SpatialConvolutionFBFFT.lua:157-164)
@@ -294,16 +298,23 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     const fbfc_conv_desc &d = p->d;
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
-    FBFC_STAGE(tm, fbfc::launch_rfft2d(N, grad_output, p->out_freq, (long)d.batch * d.out_planes,
-                                 p->info.out_h, p->info.out_w, 0, 0, s), "rfft2d(gradOutput)");
-    p->have_out = true;
-    tm.done(FBFC_STAGE_FFT_A);
-    if (!((p->reuse & FBFC_REUSE_WEIGHT) && p->have_w)) {
-        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h,
-                                     d.k_w, 0, 0, s), "rfft2d(weight)");
-        p->have_w = true;
-        tm.done(FBFC_STAGE_FFT_B);
+    const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)d.batch * d.out_planes, p->info.out_h,
+                               p->info.out_w, 0, 0};
+    const fbfc::FwdArgs fw = {weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w, 0, 0};
+    const bool need_w = !((p->reuse & FBFC_REUSE_WEIGHT) && p->have_w);
+    if (!p->timed && need_w) {
+        FBFC_TRY(fbfc::launch_rfft2d_pair(N, fgo, fw, s), "rfft2d(gradOutput, weight)");
+    } else {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fgo.in, fgo.out, fgo.planes, fgo.h, fgo.w, 0, 0, s),
+                   "rfft2d(gradOutput)");
+        tm.done(FBFC_STAGE_FFT_A);
+        if (need_w) {
+            FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fw.in, fw.out, fw.planes, fw.h, fw.w, 0, 0, s), "rfft2d(weight)");
+            tm.done(FBFC_STAGE_FFT_B);
+        }
     }
+    p->have_out = true;
+    p->have_w = true;
     float *res = p->reuse ? p->res_freq : p->in_freq;
     if (!p->reuse) p->have_in = false;
     // GI[b][p] = 1/N^2 sum_f GO[b][f] W[f][p]   (SpatialConvolutionFBFFT.lua:244-251)
@@ -325,22 +336,32 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     const fbfc_conv_desc &d = p->d;
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
+    const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)d.batch * d.out_planes, p->info.out_h,
+                               p->info.out_w, 0, 0};
+    const fbfc::FwdArgs fin = {input, p->in_freq, (long)d.batch * d.in_planes, d.in_h, d.in_w, d.pad_h, d.pad_w};
+    const bool need_go = !((p->reuse & FBFC_REUSE_OUTPUT) && p->have_out);
+    const bool need_in = !((p->reuse & FBFC_REUSE_INPUT) && p->have_in);
+    if (!p->timed && need_go && need_in) {
+        FBFC_TRY(fbfc::launch_rfft2d_pair(N, fgo, fin, s), "rfft2d(gradOutput, input)");
+    } else {
+        if (need_go) {
+            FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fgo.in, fgo.out, fgo.planes, fgo.h, fgo.w, 0, 0, s),
+                       "rfft2d(gradOutput)");
+            tm.done(FBFC_STAGE_FFT_A);
+        }
+        if (need_in) {
+            FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fin.in, fin.out, fin.planes, fin.h, fin.w, fin.padU, fin.padL, s),
+                       "rfft2d(input)");
+            tm.done(FBFC_STAGE_FFT_B);
+        }
+    }
+    p->have_out = true;
+    p->have_in = true;
     if (grad_bias != nullptr) {
-        FBFC_STAGE(tm, fbfc::launch_bias_grad(grad_output, grad_bias, scale, d.batch, d.out_planes,
-                                        p->info.out_h * p->info.out_w, p->scratch, s), "bias grad");
+        // gradBias[f] = scale * sum_b DC(gradOutput[b][f]): read off the spectrum just computed
+        FBFC_STAGE(tm, fbfc::launch_bias_grad_dc(p->out_freq, grad_bias, scale, d.batch, d.out_planes, s),
+                   "bias grad");
         tm.done(FBFC_STAGE_BIAS_GRAD);
-    }
-    if (!((p->reuse & FBFC_REUSE_OUTPUT) && p->have_out)) {
-        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, grad_output, p->out_freq, (long)d.batch * d.out_planes,
-                                     p->info.out_h, p->info.out_w, 0, 0, s), "rfft2d(gradOutput)");
-        p->have_out = true;
-        tm.done(FBFC_STAGE_FFT_A);
-    }
-    if (!((p->reuse & FBFC_REUSE_INPUT) && p->have_in)) {
-        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, input, p->in_freq, (long)d.batch * d.in_planes, d.in_h,
-                                     d.in_w, d.pad_h, d.pad_w, s), "rfft2d(input)");
-        p->have_in = true;
-        tm.done(FBFC_STAGE_FFT_B);
     }
     float *res = p->reuse ? p->res_freq : p->w_freq;
     if (!p->reuse) p->have_w = false;

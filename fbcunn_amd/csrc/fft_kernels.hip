@@ -134,16 +134,31 @@ __device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int 
 // ---------------------------------------------------------------------------------
 // forward: real (planes,h,w) -> freq [N*(N/2+1)][planes] complex
 // ---------------------------------------------------------------------------------
+// One launch can transform two tensors of the same FFT size (the two forward FFTs of a pass):
+// workgroups [0, blocks0) work on job 0, the rest on job 1.
+struct FwdJob {
+    const float *in;
+    float2 *out;
+    long planes;
+    int h, w, padU, padL, vec4;
+};
+
 template <int N>
-__global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(const float *__restrict__ in,
-                                                     float2 *__restrict__ out, long planes,
-                                                     int h, int w, int padU, int padL, int vec4)
+__global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(FwdJob job0, FwdJob job1,
+                                                                      unsigned blocks0)
 {
     using S = FftShape<N>;
     constexpr int T = S::T;
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x;
-    const long x0 = plane_group<N>(blockIdx.x) * T;
+    const bool second = blockIdx.x >= blocks0;
+    const float *__restrict__ in = second ? job1.in : job0.in;
+    float2 *__restrict__ out = second ? job1.out : job0.out;
+    const long planes = second ? job1.planes : job0.planes;
+    const int h = second ? job1.h : job0.h, w = second ? job1.w : job0.w;
+    const int padU = second ? job1.padU : job0.padU, padL = second ? job1.padL : job0.padL;
+    const int vec4 = second ? job1.vec4 : job0.vec4;
+    const long x0 = plane_group<N>(blockIdx.x - (second ? blocks0 : 0u)) * T;
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
@@ -428,10 +443,31 @@ static size_t fft_lds_bytes(int h, int w, int padU, bool inverse)
 }
 
 template <int N>
-static hipError_t launch_fwd(const float *in, float *out, long planes, int h, int w, int padU,
-                             int padL, hipStream_t s)
+static long fwd_blocks(long planes)
 {
     using S = FftShape<N>;
+    long blocks = (planes + S::T - 1) / S::T;
+    if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
+    return blocks;
+}
+
+template <int N>
+static FwdJob make_job(const float *in, float *out, long planes, int h, int w, int padU, int padL)
+{
+    using S = FftShape<N>;
+    FwdJob j;
+    j.in = in;
+    j.out = reinterpret_cast<float2 *>(out);
+    j.planes = planes;
+    j.h = h; j.w = w; j.padU = padU; j.padL = padL;
+    j.vec4 = ((reinterpret_cast<uintptr_t>(in) & 15) == 0) && (((long)S::T * h * w) % 4 == 0);
+    return j;
+}
+
+// second == nullptr: one tensor only
+template <int N>
+static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
+{
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rfft2d_kernel<N>),
@@ -439,12 +475,21 @@ static hipError_t launch_fwd(const float *in, float *out, long planes, int h, in
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    const size_t lds = fft_lds_bytes<N>(h, w, padU, false);
-    long blocks = (planes + S::T - 1) / S::T;
-    if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
-    const int vec4 = ((reinterpret_cast<uintptr_t>(in) & 15) == 0) && (((long)S::T * h * w) % 4 == 0);
-    hipLaunchKernelGGL(rfft2d_kernel<N>, dim3((unsigned)blocks), dim3(256), lds, s, in,
-                       reinterpret_cast<float2 *>(out), planes, h, w, padU, padL, vec4);
+    size_t lds = fft_lds_bytes<N>(a.h, a.w, a.padU, false);
+    const long blocks0 = fwd_blocks<N>(a.planes);
+    long blocks = blocks0;
+    const FwdJob j0 = make_job<N>(a.in, a.out, a.planes, a.h, a.w, a.padU, a.padL);
+    FwdJob j1 = j0;
+    if (second != nullptr) {
+        const size_t lds1 = fft_lds_bytes<N>(second->h, second->w, second->padU, false);
+        if (lds1 > lds) lds = lds1;
+        blocks += fwd_blocks<N>(second->planes);
+        j1 = make_job<N>(second->in, second->out, second->planes, second->h, second->w, second->padU,
+                         second->padL);
+    }
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(rfft2d_kernel<N>, dim3((unsigned)blocks), dim3(256), lds, s, j0, j1,
+                       (unsigned)blocks0);
     return hipGetLastError();
 }
 
@@ -473,17 +518,28 @@ static hipError_t launch_inv(const float *in, float *out, long planes, int h, in
 // the kernels address a frequency row with 32-bit lane offsets
 static bool planes_ok(int N, long planes) { return planes > 0 && (long)(N / 2 + 1) * planes * 8 < (1L << 31); }
 
+static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s)
+{
+    if (!planes_ok(N, a.planes) || (b != nullptr && !planes_ok(N, b->planes))) return hipErrorInvalidValue;
+    switch (N) {
+        case 8: return launch_fwd<8>(a, b, s);
+        case 16: return launch_fwd<16>(a, b, s);
+        case 32: return launch_fwd<32>(a, b, s);
+        case 64: return launch_fwd<64>(a, b, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                          int padL, hipStream_t s)
 {
-    if (!planes_ok(N, planes)) return hipErrorInvalidValue;
-    switch (N) {
-        case 8: return launch_fwd<8>(in, out, planes, h, w, padU, padL, s);
-        case 16: return launch_fwd<16>(in, out, planes, h, w, padU, padL, s);
-        case 32: return launch_fwd<32>(in, out, planes, h, w, padU, padL, s);
-        case 64: return launch_fwd<64>(in, out, planes, h, w, padU, padL, s);
-        default: return hipErrorInvalidValue;
-    }
+    const FwdArgs a = {in, out, planes, h, w, padU, padL};
+    return dispatch_fwd(N, a, nullptr, s);
+}
+
+hipError_t launch_rfft2d_pair(int N, const FwdArgs &a, const FwdArgs &b, hipStream_t s)
+{
+    return dispatch_fwd(N, a, &b, s);
 }
 
 hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,

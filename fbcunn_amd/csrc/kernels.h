@@ -9,6 +9,14 @@ namespace fbfc {
 // N in {8,16,32,64}; any other value returns hipErrorInvalidValue.
 hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                          int padL, hipStream_t s);
+// Two forward transforms of the same size in one launch (the two FFTs of a pass).
+struct FwdArgs {
+    const float *in;
+    float *out;
+    long planes;
+    int h, w, padU, padL;
+};
+hipError_t launch_rfft2d_pair(int N, const FwdArgs &a, const FwdArgs &b, hipStream_t s);
 hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                           int padL, const float *bias, int bias_period, hipStream_t s);
 
@@ -26,5 +34,9 @@ hipError_t launch_bias_add(float *out, const float *bias, int batch, int planes,
 size_t bias_grad_scratch_bytes(int batch, int planes);
 hipError_t launch_bias_grad(const float *grad_out, float *grad_bias, float scale, int batch,
                             int planes, int hw, float *scratch, hipStream_t s);
+
+// freq = frequency-major spectrum of grad_out (its first frequency row holds the plane sums)
+hipError_t launch_bias_grad_dc(const float *freq, float *grad_bias, float scale, int batch, int planes,
+                               hipStream_t s);
 
 }  // namespace fbfc

@@ -58,7 +58,7 @@ typedef struct {
     size_t input_freq_bytes;   /* Q * B * P * 8 */
     size_t weight_freq_bytes;  /* Q * F * P * 8 */
     size_t output_freq_bytes;  /* Q * B * F * 8 */
-    size_t scratch_bytes;      /* bias-gradient partial sums */
+    size_t scratch_bytes;      /* what fbfc_acc_grad_parameters_bias needs for this shape */
 } fbfc_plan_info;
 
 typedef struct fbfc_plan fbfc_plan;
