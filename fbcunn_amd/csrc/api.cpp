@@ -357,8 +357,9 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     }
     p->have_out = true;
     p->have_in = true;
-    if (grad_bias != nullptr) {
-        // gradBias[f] = scale * sum_b DC(gradOutput[b][f]): read off the spectrum just computed
+    // gradBias[f] = scale * sum_b DC(gradOutput[b][f]) is read off the spectrum just computed:
+    // its own launch when timed, otherwise a few extra workgroups of the inverse-FFT launch.
+    if (grad_bias != nullptr && p->timed) {
         FBFC_STAGE(tm, fbfc::launch_bias_grad_dc(p->out_freq, grad_bias, scale, d.batch, d.out_planes, s),
                    "bias grad");
         tm.done(FBFC_STAGE_BIAS_GRAD);
@@ -369,8 +370,14 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     FBFC_STAGE(tm, fbfc::launch_cgemm_freq(2, p->out_freq, p->in_freq, res, Q, d.out_planes, d.in_planes,
                                      d.batch, scale / ((float)N * (float)N), 0, s), "cgemm(accGrad)");
     tm.done(FBFC_STAGE_MM);
-    FBFC_STAGE(tm, fbfc::launch_irfft2d(N, res, grad_weight, (long)d.out_planes * d.in_planes, d.k_h, d.k_w,
-                                  0, 0, nullptr, 1, s), "irfft2d(gradWeight)");
+    if (grad_bias != nullptr && !p->timed) {
+        FBFC_TRY(fbfc::launch_irfft2d_bias_grad(N, res, grad_weight, (long)d.out_planes * d.in_planes, d.k_h,
+                                                d.k_w, p->out_freq, grad_bias, scale, d.batch,
+                                                d.out_planes, s), "irfft2d(gradWeight) + bias grad");
+    } else {
+        FBFC_STAGE(tm, fbfc::launch_irfft2d(N, res, grad_weight, (long)d.out_planes * d.in_planes, d.k_h,
+                                            d.k_w, 0, 0, nullptr, 1, s), "irfft2d(gradWeight)");
+    }
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();
 }

@@ -1,0 +1,34 @@
+// Bias gradient from the spectrum of gradOutput.
+//
+// The zero-frequency bin of plane (b, f) is sum_{r,c} gradOutput[b][f][r][c], so
+// gradBias[f] = scale * sum_b Re dc[b][f] with dc the first frequency row of the
+// frequency-major spectrum (batch x planes complex numbers).  One 256-lane workgroup
+// handles 64 planes x 4 batch slices; `part` is 4 x 64 floats of LDS.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace fbfc {
+
+struct BiasGradJob {
+    const float2 *dc;   // first frequency row of FFT(gradOutput); nullptr = no job
+    float *grad_bias;
+    float scale;
+    int batch, planes;
+};
+
+__device__ __forceinline__ void bias_grad_dc_body(const BiasGradJob &j, unsigned block, float (*part)[64])
+{
+    const int fl = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int f = (int)block * 64 + fl;
+    float acc = 0.0f;
+    if (f < j.planes)
+        for (int b = slice; b < j.batch; b += 4) acc += j.dc[(long)b * j.planes + f].x;
+    part[slice][fl] = acc;
+    __syncthreads();
+    if (slice == 0 && f < j.planes)
+        j.grad_bias[f] = ((part[0][fl] + part[1][fl]) + (part[2][fl] + part[3][fl])) * j.scale;
+}
+
+inline unsigned bias_grad_dc_blocks(int planes) { return (unsigned)((planes + 63) / 64); }
+
+}  // namespace fbfc

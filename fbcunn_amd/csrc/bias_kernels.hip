@@ -10,6 +10,7 @@
 // the partial sums in a fixed order, so the result is deterministic.
 #include <hip/hip_runtime.h>
 
+#include "bias_dc.h"
 #include "kernels.h"
 
 namespace fbfc {
@@ -63,31 +64,19 @@ __global__ __launch_bounds__(256) void bias_grad_final_kernel(const float *__res
     grad_bias[f] = acc * scale;
 }
 
-// Inside accGradParameters the spectrum of gradOutput is already in HBM, and the zero-frequency
-// bin of plane (b, f) IS sum_{r,c} gradOutput[b][f][r][c]: the bias gradient is a column sum of
-// the first frequency row, B*F complex numbers instead of B*F*oH*oW floats.
-// dc = freq[0] viewed as (batch x planes) complex; workgroup = 64 planes x 4 batch slices.
-__global__ __launch_bounds__(256) void bias_grad_dc_kernel(const float2 *__restrict__ dc,
-                                                           float *__restrict__ grad_bias,
-                                                           float scale, int batch, int planes)
+// Stand-alone launch of the zero-frequency-row bias gradient (see bias_dc.h); the
+// accGradParameters pass normally runs the same body inside its inverse-FFT launch.
+__global__ __launch_bounds__(256) void bias_grad_dc_kernel(BiasGradJob job)
 {
     __shared__ float part[4][64];
-    const int fl = threadIdx.x & 63, slice = threadIdx.x >> 6;
-    const int f = blockIdx.x * 64 + fl;
-    float acc = 0.0f;
-    if (f < planes)
-        for (int b = slice; b < batch; b += 4) acc += dc[(long)b * planes + f].x;
-    part[slice][fl] = acc;
-    __syncthreads();
-    if (slice == 0 && f < planes)
-        grad_bias[f] = ((part[0][fl] + part[1][fl]) + (part[2][fl] + part[3][fl])) * scale;
+    bias_grad_dc_body(job, blockIdx.x, part);
 }
 
 hipError_t launch_bias_grad_dc(const float *freq, float *grad_bias, float scale, int batch, int planes,
                                hipStream_t s)
 {
-    hipLaunchKernelGGL(bias_grad_dc_kernel, dim3((planes + 63) / 64), dim3(256), 0, s,
-                       reinterpret_cast<const float2 *>(freq), grad_bias, scale, batch, planes);
+    BiasGradJob job = {reinterpret_cast<const float2 *>(freq), grad_bias, scale, batch, planes};
+    hipLaunchKernelGGL(bias_grad_dc_kernel, dim3(bias_grad_dc_blocks(planes)), dim3(256), 0, s, job);
     return hipGetLastError();
 }
 

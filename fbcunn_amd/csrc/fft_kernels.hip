@@ -23,6 +23,7 @@
 // The inverse kernel is the mirror image and adds the bias while cropping.
 #include <hip/hip_runtime.h>
 
+#include "bias_dc.h"
 #include "fft_regs.h"
 #include "kernels.h"
 
@@ -302,13 +303,20 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void irfft2d_kernel(const flo
                                                       float *__restrict__ out, long planes,
                                                       int h, int w, int padU, int padL,
                                                       const float *__restrict__ bias,
-                                                      int bias_period, int vec4)
+                                                      int bias_period, int vec4, BiasGradJob bgrad,
+                                                      unsigned bgrad_blocks)
 {
     using S = FftShape<N>;
     constexpr int T = S::T;
     extern __shared__ __align__(16) float smem[];
+    if (blockIdx.x < bgrad_blocks) {
+        // an independent small job riding on this launch: the bias gradient of the same pass
+        // (1 KB of the dynamic LDS, which is never smaller than one tile row pair)
+        bias_grad_dc_body(bgrad, blockIdx.x, reinterpret_cast<float (*)[64]>(smem));
+        return;
+    }
     const int tid = threadIdx.x;
-    const long x0 = plane_group<N>(blockIdx.x) * T;
+    const long x0 = plane_group<N>(blockIdx.x - bgrad_blocks) * T;
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
@@ -495,7 +503,8 @@ static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_
 
 template <int N>
 static hipError_t launch_inv(const float *in, float *out, long planes, int h, int w, int padU,
-                             int padL, const float *bias, int bias_period, hipStream_t s)
+                             int padL, const float *bias, int bias_period, const BiasGradJob &bgrad,
+                             hipStream_t s)
 {
     using S = FftShape<N>;
     static bool attr_done = false;
@@ -509,9 +518,10 @@ static hipError_t launch_inv(const float *in, float *out, long planes, int h, in
     long blocks = (planes + S::T - 1) / S::T;
     if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
     const int vec4 = ((reinterpret_cast<uintptr_t>(out) & 15) == 0) && (((long)S::T * h * w) % 4 == 0);
-    hipLaunchKernelGGL(irfft2d_kernel<N>, dim3((unsigned)blocks), dim3(256), lds, s,
+    const unsigned bblocks = (bgrad.dc != nullptr) ? bias_grad_dc_blocks(bgrad.planes) : 0u;
+    hipLaunchKernelGGL(irfft2d_kernel<N>, dim3((unsigned)blocks + bblocks), dim3(256), lds, s,
                        reinterpret_cast<const float2 *>(in), out, planes, h, w, padU, padL, bias,
-                       bias_period > 0 ? bias_period : 1, vec4);
+                       bias_period > 0 ? bias_period : 1, vec4, bgrad, bblocks);
     return hipGetLastError();
 }
 
@@ -542,17 +552,33 @@ hipError_t launch_rfft2d_pair(int N, const FwdArgs &a, const FwdArgs &b, hipStre
     return dispatch_fwd(N, a, &b, s);
 }
 
-hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
-                          int padL, const float *bias, int bias_period, hipStream_t s)
+static hipError_t dispatch_inv(int N, const float *in, float *out, long planes, int h, int w, int padU,
+                               int padL, const float *bias, int bias_period, const BiasGradJob &bgrad,
+                               hipStream_t s)
 {
     if (!planes_ok(N, planes)) return hipErrorInvalidValue;
     switch (N) {
-        case 8: return launch_inv<8>(in, out, planes, h, w, padU, padL, bias, bias_period, s);
-        case 16: return launch_inv<16>(in, out, planes, h, w, padU, padL, bias, bias_period, s);
-        case 32: return launch_inv<32>(in, out, planes, h, w, padU, padL, bias, bias_period, s);
-        case 64: return launch_inv<64>(in, out, planes, h, w, padU, padL, bias, bias_period, s);
+        case 8: return launch_inv<8>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
+        case 16: return launch_inv<16>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
+        case 32: return launch_inv<32>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
+        case 64: return launch_inv<64>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
+                          int padL, const float *bias, int bias_period, hipStream_t s)
+{
+    const BiasGradJob none = {nullptr, nullptr, 0.0f, 0, 0};
+    return dispatch_inv(N, in, out, planes, h, w, padU, padL, bias, bias_period, none, s);
+}
+
+hipError_t launch_irfft2d_bias_grad(int N, const float *in, float *out, long planes, int h, int w,
+                                    const float *go_freq, float *grad_bias, float scale, int batch,
+                                    int out_planes, hipStream_t s)
+{
+    const BiasGradJob job = {reinterpret_cast<const float2 *>(go_freq), grad_bias, scale, batch, out_planes};
+    return dispatch_inv(N, in, out, planes, h, w, 0, 0, nullptr, 1, job, s);
 }
 
 }  // namespace fbfc

@@ -20,6 +20,12 @@ hipError_t launch_rfft2d_pair(int N, const FwdArgs &a, const FwdArgs &b, hipStre
 hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                           int padL, const float *bias, int bias_period, hipStream_t s);
 
+// Inverse transform (no padding offset, no bias add) that also carries the pass's bias gradient:
+// grad_bias[f] = scale * sum_b Re go_freq[0][b][f] (go_freq = spectrum of gradOutput).
+hipError_t launch_irfft2d_bias_grad(int N, const float *in, float *out, long planes, int h, int w,
+                                    const float *go_freq, float *grad_bias, float scale, int batch,
+                                    int out_planes, hipStream_t s);
+
 // cgemm_kernels.hip ------------------------------------------------------------
 // mode 0: C[m][n] (+)= alpha * sum_k A[m][k] * conj(B[n][k])   A (m x k), B (n x k)
 // mode 1: C[m][n] (+)= alpha * sum_k A[m][k] * B[k][n]         A (m x k), B (k x n)
