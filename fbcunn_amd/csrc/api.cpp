@@ -30,7 +30,7 @@ int fail_hip(hipError_t e, const char *what)
 }
 
 constexpr int kMinFft = 8;
-constexpr int kMaxFft = 64;
+constexpr int kMaxFft = 128;
 
 // fbcunn/SpatialConvolutionFFT.lua:875-882 (2^i, i = 1..10)
 int next_power_of_2(int v)
@@ -81,7 +81,7 @@ int plan_query(const fbfc_conv_desc *d, fbfc_plan_info *info)
     return FBFC_OK;
 }
 
-bool fft_size_ok(int n) { return n == 8 || n == 16 || n == 32 || n == 64; }
+bool fft_size_ok(int n) { return n == 8 || n == 16 || n == 32 || n == 64 || n == 128; }
 
 }  // namespace
 

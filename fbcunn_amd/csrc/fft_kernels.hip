@@ -38,9 +38,11 @@ struct FftShape {
     // Phases: the LDS tile holds NH2/PH of the tile columns at a time and the input /
     // output staging area T/PH planes at a time, so that two workgroups fit one CU's
     // 160 KB LDS even for N = 64 (a full 8-plane tile would need 117 KB).
-    static constexpr int PH = (N >= 64) ? 2 : 1;
+    static constexpr int PH = (N >= 128) ? 4 : (N >= 64) ? 2 : 1;
     static constexpr int KXP = NH2 / PH;    // tile columns per phase
     static constexpr int TP = T / PH;       // planes per staging round
+    // waves per SIMD the register budget is sized for (N = 128 keeps 256 values per lane)
+    static constexpr int MIN_WAVES = (N >= 128) ? 1 : PH;
     // padding (in complex elements) between tile rows: keeps the T-lane groups
     // of one wave on different LDS banks when T*8 bytes is below 128
     static constexpr int ROWPAD = (T * 8 < 128) ? (64 / 8) / 2 : 0;
@@ -145,7 +147,7 @@ struct FwdJob {
 };
 
 template <int N>
-__global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(FwdJob job0, FwdJob job1,
+__global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(FwdJob job0, FwdJob job1,
                                                                       unsigned blocks0)
 {
     using S = FftShape<N>;
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(256, FftShape<N>::PH) void rfft2d_kernel(FwdJob job
 // real[r][s] = y[r+padU][s+padL] (+ bias[plane % bias_period])
 // ---------------------------------------------------------------------------------
 template <int N>
-__global__ __launch_bounds__(256, FftShape<N>::PH) void irfft2d_kernel(const float2 *__restrict__ in,
+__global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void irfft2d_kernel(const float2 *__restrict__ in,
                                                       float *__restrict__ out, long planes,
                                                       int h, int w, int padU, int padL,
                                                       const float *__restrict__ bias,
@@ -536,6 +538,7 @@ static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStr
         case 16: return launch_fwd<16>(a, b, s);
         case 32: return launch_fwd<32>(a, b, s);
         case 64: return launch_fwd<64>(a, b, s);
+        case 128: return launch_fwd<128>(a, b, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -562,6 +565,7 @@ static hipError_t dispatch_inv(int N, const float *in, float *out, long planes, 
         case 16: return launch_inv<16>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
         case 32: return launch_inv<32>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
         case 64: return launch_inv<64>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
+        case 128: return launch_inv<128>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
         default: return hipErrorInvalidValue;
     }
 }

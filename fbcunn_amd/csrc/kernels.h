@@ -6,7 +6,7 @@
 namespace fbfc {
 
 // fft_kernels.hip ------------------------------------------------------------
-// N in {8,16,32,64}; any other value returns hipErrorInvalidValue.
+// N in {8,16,32,64,128}; any other value returns hipErrorInvalidValue.
 hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                          int padL, hipStream_t s);
 // Two forward transforms of the same size in one launch (the two FFTs of a pass).

@@ -72,7 +72,8 @@ const char *fbfc_last_error(void);
  * Validates the descriptor the way the module constructor and the FFT-size
  * choice do (stride 1: SpatialConvolutionFFT.lua:176, SpatialConvolutionFBFFT.lua:60-61;
  * pad < kernel: SpatialConvolutionFBFFT.lua:93-95; nextPowerOf2: SpatialConvolutionFFT.lua:875-882)
- * and fills *info.  FFT sizes above 64 are FBFC_ERR_UNSUPPORTED_SIZE. */
+ * and fills *info.  FFT sizes above 128 are FBFC_ERR_UNSUPPORTED_SIZE (the reference's
+ * fbfft stops at 128 as well); sizes below 8 run on an 8 x 8 canvas. */
 int fbfc_plan_query(const fbfc_conv_desc *desc, fbfc_plan_info *info);
 
 /* Plans -----------------------------------------------------------------------
@@ -133,7 +134,7 @@ int fbfc_plan_stage_ms(const fbfc_plan *plan, float *ms, int n);
  * Replaces FFTWrapper_fft with fbfft (src/fft/FFTWrapperLua.cpp:209-272 ->
  * fbfft2dHost, src/fft/FBFFTHost.cpp:39-116): batched 2-D real-to-complex FFT of
  * `planes` h x w planes, each implicitly zero-padded into an N x N canvas at
- * row pad_u, column pad_l.  N in {8,16,32,64}.  Output is frequency-major. */
+ * row pad_u, column pad_l.  N in {8,16,32,64,128}.  Output is frequency-major. */
 int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l,
                int fft_size, float *freq, void *stream);
 

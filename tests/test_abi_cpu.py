@@ -38,6 +38,7 @@ def _q(**kw):
     (dict(batch=4, in_planes=16, out_planes=16, in_h=32, in_w=32, k_h=5, k_w=5, pad_h=0, pad_w=0), 32, 544, 28),
     (dict(in_h=3, in_w=3, k_h=2, k_w=2, pad_h=0, pad_w=0), 8, 40, 2),      # tiny: canvas rounded up to 8
     (dict(in_h=16, in_w=9, k_h=3, k_w=3, pad_h=1, pad_w=0), 32, 544, 16),   # square canvas from the larger side
+    (dict(in_h=100, in_w=90, k_h=5, k_w=5, pad_h=2, pad_w=2), 128, 8320, 100),
 ])
 def test_plan_sizes(kw, n, q, o):
     info = _q(**kw)
@@ -59,7 +60,7 @@ def test_plan_buffer_bytes_match_reference_layout():
     (dict(pad_w=5), _lib.ERR_INVALID_ARGUMENT, "Padding must be smaller than kernel"),
     (dict(batch=0), _lib.ERR_INVALID_ARGUMENT, "positive"),
     (dict(in_h=2, in_w=2, k_h=5, k_w=5, pad_h=0, pad_w=0), _lib.ERR_INVALID_ARGUMENT, "kernel larger"),
-    (dict(in_h=100, in_w=100), _lib.ERR_UNSUPPORTED_SIZE, "not supported"),
+    (dict(in_h=200, in_w=100), _lib.ERR_UNSUPPORTED_SIZE, "not supported"),
     (dict(in_h=2000, in_w=5), _lib.ERR_UNSUPPORTED_SIZE, "Too large"),
 ])
 def test_plan_rejections(kw, code, text):

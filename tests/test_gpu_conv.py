@@ -69,6 +69,7 @@ PROBLEMS = [
     (2, 3, 4, 3, 5, 10, 17, 2, 0), (2, 3, 4, 6, 2, 20, 9, 0, 1), (1, 2, 3, 4, 4, 40, 23, 3, 3),  # rectangular
     (3, 70, 66, 3, 3, 12, 12, 1, 1),                                                     # ragged GEMM tiles
     (5, 2, 3, 7, 7, 7, 7, 6, 6),                                                          # pad = k-1 (full conv)
+    (2, 3, 4, 5, 5, 100, 90, 2, 2), (1, 2, 2, 11, 11, 118, 118, 5, 5),                    # FFT size 128
 ]
 
 
@@ -202,5 +203,5 @@ def test_module_argument_errors(nn):
     with pytest.raises(TypeError):
         net.updateOutput(torch.zeros(1, 3, 8, 8))               # not on the GPU
     with pytest.raises(nn.FbfcError) as e:
-        net.updateOutput(torch.zeros(1, 3, 100, 100, device="cuda"))   # FFT size 128 not built
+        net.updateOutput(torch.zeros(1, 3, 200, 200, device="cuda"))   # FFT size 256: beyond fbfft's 128
     assert e.value.code == 2
