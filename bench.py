@@ -62,6 +62,22 @@ KERNEL_OF_STAGE = {"fft_a": "rfft2d_kernel", "fft_b": "rfft2d_kernel", "mm": "cg
                    "ifft": "irfft2d_kernel", "bias_grad": "bias_grad_dc_kernel"}
 
 
+def mm_kernel_name(pass_, q, m, n, k):
+    """Which contraction kernel the library picks (the rule of launch_mode in
+    fbcunn_amd/csrc/cgemm_kernels.hip), so that the stage table names the kernel
+    a rocprofv3 trace of the same run shows."""
+    mode = {"fprop": 0, "bprop": 1, "accgrad": 2}[pass_]
+    if m % 32 == 0 and n % 32 == 0 and k % 16 == 0:
+        tot32 = q * (m // 32) * (n // 32)
+        if tot32 < 4096 and k % 64 == 0:
+            return "cgemm_splitk_kernel<%d, 4>" % mode
+        if tot32 < 8192 and k % 32 == 0:
+            return "cgemm_splitk_kernel<%d, 2>" % mode
+        if mode != 0:
+            return "cgemm_splitk_kernel<%d, 1>" % mode
+    return "cgemm_freq_kernel<%d>" % mode
+
+
 def make_layer(nn, torch, synth, cfg):
     B, P, F, H, k, pad, _, wstd, seed = cfg
     o = H + 2 * pad - k + 1
@@ -135,7 +151,8 @@ def measure_config(nn, torch, synth, name, steps, warmup):
                                       "peak": HBM_PEAK_GBS, "frac": ach / HBM_PEAK_GBS}
             else:
                 ach = spec[1] / (ms_s * 1e-3) / 1e12
-                entry["stages"][s] = {"kernel": KERNEL_OF_STAGE[s], "ms": ms_s, "bound": "mfma",
+                mnk = {"fprop": (B, F, P), "bprop": (B, P, F), "accgrad": (F, P, B)}[p]
+                entry["stages"][s] = {"kernel": mm_kernel_name(p, q, *mnk), "ms": ms_s, "bound": "mfma",
                                       "flops": spec[1], "bytes": spec[2], "achieved": ach,
                                       "unit": "TFLOP/s", "peak": MFMA_FP32_PEAK_TF,
                                       "frac": ach / MFMA_FP32_PEAK_TF,
@@ -169,6 +186,38 @@ def measure_fft_round_trip(nn, torch, synth, steps, warmup):
         out[name] = {"ms": ms, "bytes": nbytes, "achieved": ach, "unit": "GB/s", "peak": HBM_PEAK_GBS,
                      "frac": ach / HBM_PEAK_GBS}
     return out
+
+
+def measure_reuse_step(nn, torch, synth, steps, warmup):
+    """The same training step with memoryReuseAll (bprop reuses FFT(weight), accGrad reuses
+    FFT(gradOutput) and FFT(input)): 3 forward FFTs per step instead of 6."""
+    cfg = CONFIGS[MAIN]
+    B, P, F, H, k, pad, passes, wstd, seed = cfg
+    o = H + 2 * pad - k + 1
+    net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad, "all")
+    net.weight.copy_(torch.from_numpy(synth.normal(seed, (F, P, k, k), 0.0, wstd, stream=1)).cuda())
+    net.bias.zero_()
+    x = torch.from_numpy(synth.uniform(seed, (B, P, H, H), stream=0)).cuda()
+    g = torch.from_numpy(synth.uniform(seed, (B, F, o, o), stream=3)).cuda()
+    ms = time_loop(torch, lambda: [run_pass(net, x, g, p) for p in passes], steps, warmup)
+    net.cleanupBuffers()
+    return {"ms_per_step": ms, "effective_tflops": 3 * 2.0 * B * F * P * o * o * k * k / (ms * 1e-3) / 1e12}
+
+
+def measure_copy_bandwidth(torch):
+    """A plain 256 MiB device-to-device copy: what HBM delivers to a trivial kernel on this box."""
+    a = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+    b = torch.empty_like(a)
+    for _ in range(3):
+        b.copy_(a)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        b.copy_(a)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / 10
+    return {"ms": ms, "GBps_read_plus_write": 2 * a.numel() * 4 / (ms * 1e-3) / 1e9}
 
 
 def cpu_baseline(synth):
@@ -251,6 +300,8 @@ def main():
         "roofline": roofline,
         "stages": {k: v["stages"] for k, v in main_res["passes"].items()},
     }
+    line["reuse_all_step"] = measure_reuse_step(nn, torch, synth, args.steps, args.warmup)
+    line["copy_256MiB"] = measure_copy_bandwidth(torch)
     if args.all_configs:
         others = {}
         for name in CONFIGS:
