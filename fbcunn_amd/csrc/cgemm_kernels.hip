@@ -211,7 +211,8 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
 // is a quarter block (9 per SIMD for config 4).  Operands go straight from global memory into
 // the MFMA operand registers (each lane loads exactly the k' it feeds: 64 contiguous bytes of
 // a K-contiguous row, or one complex per row of a row-contiguous operand); LDS is used only
-// to add the four partial accumulators.  Preconditions: M % 32 == N % 32 == 0, K % 64 == 0.
+// to add the partial accumulators.  Preconditions: M % 32 == N % 32 == 0, K % (16 * SK) == 0
+// (SK = waves that share one block: 4, 2 or 1; with SK = 1 a workgroup is four independent blocks).
 // ---------------------------------------------------------------------------------------
 template <int MODE>
 __device__ __forceinline__ void splitk_load(const float2 *__restrict__ Aq, const float2 *__restrict__ Bq,
@@ -314,22 +315,33 @@ __global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restr
     for (int r = 0; r < 16; ++r) { cre[r] = 0.f; cim[r] = 0.f; }
 
     if (live) {
-        float a0[16], b0[16], a1[16], b1[16];
-        splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg, h, a0, b0);
-        int kt = 0;
-        for (; kt + 1 < nkt; kt += 2) {
-            splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * (kt + 1), h, a1, b1);
-            __builtin_amdgcn_sched_barrier(0);
-            splitk_mfma<MODE>(a0, b0, cre, cim);
-            __builtin_amdgcn_sched_barrier(0);
-            // the last prefetch of an even count re-reads the final tile and is not used
-            const int knext = (kt + 2 < nkt) ? kt + 2 : kt + 1;
-            splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * knext, h, a0, b0);
-            __builtin_amdgcn_sched_barrier(0);
-            splitk_mfma<MODE>(a1, b1, cre, cim);
-            __builtin_amdgcn_sched_barrier(0);
+        if constexpr (SK == 1) {
+            // long K loop per wave: explicit register double buffering, loads pinned ahead of the MFMAs
+            float a0[16], b0[16], a1[16], b1[16];
+            splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg, h, a0, b0);
+            int kt = 0;
+            for (; kt + 1 < nkt; kt += 2) {
+                splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * (kt + 1), h, a1, b1);
+                __builtin_amdgcn_sched_barrier(0);
+                splitk_mfma<MODE>(a0, b0, cre, cim);
+                __builtin_amdgcn_sched_barrier(0);
+                // the last prefetch of an even count re-reads the final tile and is not used
+                const int knext = (kt + 2 < nkt) ? kt + 2 : kt + 1;
+                splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * knext, h, a0, b0);
+                __builtin_amdgcn_sched_barrier(0);
+                splitk_mfma<MODE>(a1, b1, cre, cim);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (kt < nkt) splitk_mfma<MODE>(a0, b0, cre, cim);
+        } else {
+            // one to four K-tiles per wave: the compiler interleaves each tile's loads with the
+            // previous tile's MFMAs, and at about 64 registers per lane five workgroups share a CU
+            float a[16], b[16];
+            for (int kt = 0; kt < nkt; ++kt) {
+                splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * kt, h, a, b);
+                splitk_mfma<MODE>(a, b, cre, cim);
+            }
         }
-        if (kt < nkt) splitk_mfma<MODE>(a0, b0, cre, cim);
     }
 
     if constexpr (SK == 1) {
