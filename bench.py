@@ -67,14 +67,19 @@ def mm_kernel_name(pass_, q, m, n, k):
     fbcunn_amd/csrc/cgemm_kernels.hip), so that the stage table names the kernel
     a rocprofv3 trace of the same run shows."""
     mode = {"fprop": 0, "bprop": 1, "accgrad": 2}[pass_]
+    tiles64 = q * ((m + 63) // 64) * ((n + 63) // 64)
+    direct_ok = m % 64 == 0 and n % 64 == 0 and k % 16 == 0
+    if direct_ok and tiles64 >= 4 * 256:
+        return "cgemm_ldsdirect_kernel<%d>" % mode
     if m % 32 == 0 and n % 32 == 0 and k % 16 == 0:
         tot32 = q * (m // 32) * (n // 32)
         if tot32 < 4096 and k % 64 == 0:
             return "cgemm_splitk_kernel<%d, 4>" % mode
         if tot32 < 8192 and k % 32 == 0:
             return "cgemm_splitk_kernel<%d, 2>" % mode
-        if mode != 0:
-            return "cgemm_splitk_kernel<%d, 1>" % mode
+        return "cgemm_splitk_kernel<%d, 1>" % mode
+    if direct_ok:
+        return "cgemm_ldsdirect_kernel<%d>" % mode
     return "cgemm_freq_kernel<%d>" % mode
 
 

@@ -203,6 +203,164 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
 }
 
 // ---------------------------------------------------------------------------------------
+// LDS-direct variant of the tiled kernel (M % 64 == N % 64 == 0, K % 16 == 0).
+//
+// Operand tiles go from global memory straight into LDS with global_load_lds_dwordx4: no
+// staging registers, no ds_write, and the returning data does not compete with the MFMAs for
+// the vector register file (measured on this chip: with the same bytes per flop a MFMA loop
+// fed by register loads sustains about 100 TFLOP/s, fed by LDS-direct loads about 125).
+// One such instruction writes 64 lanes x 16 bytes to 1 KB of consecutive LDS, lane l at
+// base + 16 l, each lane from its own global address; the tile layout in LDS is therefore
+// chosen through which 16-byte chunk each lane fetches:
+//   K-contiguous tile [64 rows][8 chunks]: one instruction = 8 rows; lane (r, c') fetches chunk
+//     c = c' ^ r of row r, so that the 16-byte reads "chunk c of 8 consecutive rows" hit 8
+//     different bank groups (XOR swizzle instead of row padding);
+//   row-contiguous tile [16 k][32 chunks]: one instruction = 2 rows, stored as they lie.
+// ---------------------------------------------------------------------------------------
+template <bool KC>
+__device__ __forceinline__ void lds_direct_tile(const float2 *__restrict__ Mq, int ld, int r0, int c0,
+                                                float *lds, int wave, int lane)
+{
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int blk = j * 4 + wave;  // 1 KB block of the 8 KB tile
+        const float2 *g;
+        if (KC) {  // rows r0 + 8 blk .. +7, complex k c0 .. c0+15
+            const int rl = lane >> 3, cs = lane & 7;
+            g = Mq + (long)(r0 + 8 * blk + rl) * ld + c0 + 2 * (cs ^ rl);
+        } else {   // k rows r0 + 2 blk, +1; complex columns c0 .. c0+63
+            const int kl = lane >> 5, cs = lane & 31;
+            g = Mq + (long)(r0 + 2 * blk + kl) * ld + c0 + 2 * cs;
+        }
+        __builtin_amdgcn_global_load_lds(
+            (const void __attribute__((address_space(1))) *)g,
+            (void __attribute__((address_space(3))) *)(lds + blk * 256), 16, 0, 0);
+    }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void cgemm_ldsdirect_kernel(const float2 *__restrict__ A,
+                                                              const float2 *__restrict__ B,
+                                                              float2 *__restrict__ C, int M, int N,
+                                                              int K, float alpha, int accumulate,
+                                                              int tilesM, int tilesN, int total_wgs,
+                                                              int chunk)
+{
+    constexpr bool A_KC = (MODE != 2);
+    constexpr bool B_KC = (MODE == 0);
+    constexpr int TILE = 64 * KT * 2;  // floats per operand tile (8 KB)
+    __shared__ __align__(16) float As[2][TILE];
+    __shared__ __align__(16) float Bs[2][TILE];
+
+    const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
+    if (wg >= total_wgs) return;
+    const int tiles = tilesM * tilesN;
+    const int q = wg / tiles;
+    const int tile = wg - q * tiles;
+    const int m0 = (tile / tilesN) * BM;
+    const int n0 = (tile % tilesN) * BN;
+    const float2 *Aq = A + (long)q * M * K;
+    const float2 *Bq = B + (long)q * N * K;
+    float2 *Cq = C + (long)q * M * N;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, h = lane >> 5;
+
+    floatx16 cre, cim;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { cre[r] = 0.f; cim[r] = 0.f; }
+
+    const int nk = K / KT;
+    auto issue = [&](int kt, int buf) {
+        const int k0 = kt * KT;
+        if (A_KC) lds_direct_tile<true>(Aq, K, m0, k0, As[buf], wave, lane);   // A[m][k]
+        else      lds_direct_tile<false>(Aq, M, k0, m0, As[buf], wave, lane);  // A[k][m]
+        if (B_KC) lds_direct_tile<true>(Bq, K, n0, k0, Bs[buf], wave, lane);   // B[n][k]
+        else      lds_direct_tile<false>(Bq, N, k0, n0, Bs[buf], wave, lane);  // B[k][n]
+    };
+
+    issue(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    __syncthreads();
+
+    const int arow = 32 * wm + li, bcol = 32 * wn + li;
+    // swizzled position of 16-byte chunk c of a K-contiguous row: 8-row block, row in block, c ^ row
+    const int a_blk = (arow >> 3) * 256 + (arow & 7) * 32, a_x = arow & 7;
+    const int b_blk = (bcol >> 3) * 256 + (bcol & 7) * 32, b_x = bcol & 7;
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) issue(kt + 1, buf ^ 1);  // asynchronous: lands while this tile is multiplied
+
+        const float *as = As[buf];
+        const float *bs = Bs[buf];
+        if (MODE == 0) {
+            float a[16], b[16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 va = *reinterpret_cast<const float4 *>(as + a_blk + (((4 * h + j) ^ a_x) << 2));
+                const float4 vb = *reinterpret_cast<const float4 *>(bs + b_blk + (((4 * h + j) ^ b_x) << 2));
+                a[4 * j] = va.x; a[4 * j + 1] = va.y; a[4 * j + 2] = va.z; a[4 * j + 3] = va.w;
+                b[4 * j] = vb.x; b[4 * j + 1] = vb.y; b[4 * j + 2] = vb.z; b[4 * j + 3] = vb.w;
+            }
+#pragma unroll
+            for (int s = 0; s < 16; s += 2) {
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], -b[s + 1], cim, 0, 0, 0);
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s + 1], b[s + 1], cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s + 1], b[s], cim, 0, 0, 0);
+            }
+        } else if (MODE == 1) {
+            float a[16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 va = *reinterpret_cast<const float4 *>(as + a_blk + (((4 * h + j) ^ a_x) << 2));
+                a[4 * j] = va.x; a[4 * j + 1] = va.y; a[4 * j + 2] = va.z; a[4 * j + 3] = va.w;
+            }
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDM + 2 * bcol);
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.x, cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.y, cim, 0, 0, 0);
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], -vb.y, cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], vb.x, cim, 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                // half-wave h owns k = 8h + kk: both components of conj(A)[k][arow] and B[k][bcol]
+                const float2 va = *reinterpret_cast<const float2 *>(as + (8 * h + kk) * LDM + 2 * arow);
+                const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDM + 2 * bcol);
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(va.x, vb.x, cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(va.x, vb.y, cim, 0, 0, 0);
+                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(va.y, vb.y, cre, 0, 0, 0);
+                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(va.y, -vb.x, cim, 0, 0, 0);
+            }
+        }
+        if (kt + 1 < nk) {
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's share of the next tile is in LDS
+            __syncthreads();                     // ... and everyone's; nobody still reads the other buffer
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int row = m0 + 32 * wm + 8 * (r / 4) + 4 * h + (r % 4);
+        const int col = n0 + 32 * wn + li;
+        float2 v = make_float2(alpha * cre[r], alpha * cim[r]);
+        float2 *dst = Cq + (long)row * N + col;
+        if (accumulate) {
+            const float2 o = *dst;
+            v.x += o.x;
+            v.y += o.y;
+        }
+        *dst = v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Split-K kernel for small problems (few 64x64 tiles per CU).
 //
 // With only a handful of output tiles per SIMD, whole tiles cannot be balanced over the 1024
@@ -407,7 +565,8 @@ static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_
     return hipGetLastError();
 }
 
-// FBFC_CGEMM_SPLITK = 0 (LDS-tiled kernel), 1, 2 or 4 forces a kernel variant (for measurements).
+// FBFC_CGEMM_SPLITK forces a kernel variant (for measurements): 0 = register-staged LDS tiles,
+// 8 = LDS-direct tiles, 1 / 2 / 4 = register-fed kernel with that many waves per block.
 static int splitk_override()
 {
     static int v = -2;
@@ -425,22 +584,35 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
     const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
     const long total = (long)n_freq * tilesM * tilesN;
     if (total <= 0 || total > 0x7fffff00L) return hipErrorInvalidValue;
-    // Register-fed kernel when the shape allows it (blocks of 32, K-tiles of 16, 16-byte aligned
-    // operands).  The fewer blocks there are per SIMD, the more waves share one block's K range.
+    // Kernel choice (measured on MI355X):
+    //  * at least 4 full 64x64 tiles per CU and 64-aligned M, N: LDS-direct tiles;
+    //  * otherwise, if M, N are multiples of 32 and K of 16: the register-fed kernel, with more
+    //    waves sharing one block's K range the fewer blocks there are per SIMD;
+    //  * anything else: register-staged LDS tiles with bounds checks.
     const bool aligned16 = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
+    const int force = splitk_override();
+    const bool direct_ok = (m % 64) == 0 && (n % 64) == 0 && (k % 16) == 0 && aligned16;
     const long tot32 = (long)n_freq * (m / 32) * (n / 32);
-    if ((m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 && tot32 * 4 < 0x7fffff00L) {
-        const int force = splitk_override();
+    const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && total >= 4 * 256));
+    if (!prefer_direct && (m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 &&
+        tot32 * 4 < 0x7fffff00L) {
         int sk = 0;
-        if (force >= 0) sk = force;
+        if (force >= 0) sk = (force == 8) ? 0 : force;
         else if (tot32 < 4 * 1024 && (k % 64) == 0) sk = 4;
         else if (tot32 < 8 * 1024 && (k % 32) == 0) sk = 2;
-        else if (MODE != 0) sk = 1;   // K-contiguous operands on both sides do as well through LDS
+        else sk = 1;
         if (sk == 4 && (k % 64) == 0) return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
         if (sk == 2 && (k % 32) == 0) return launch_splitk<MODE, 2>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
         if (sk == 1) return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
     }
     const int chunk = (int)((total + 7) / 8);
+    if (direct_ok && force != 0) {
+        hipLaunchKernelGGL(cgemm_ldsdirect_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
+                           reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
+                           reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
+                           (int)total, chunk);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                        reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
