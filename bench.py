@@ -58,6 +58,15 @@ def stage_model(cfg, pass_, n, q):
             "ifft": ("hbm", fft(F * P, k))}
 
 
+# HBM bytes per launch at the main workload, from the committed rocprofv3 --pmc runs
+# (profiles/hbm_traffic_all_configs.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, the
+# factors a 256 MiB device copy gives for the same counters (--calibrate-copy).
+MEASURED_TRAFFIC_MAIN = {
+    "cgemm_splitk_kernel<0, 4>": (18462 * 2.0 + 18432) * 1024,
+    "cgemm_splitk_kernel<1, 4>": (18462 * 2.0 + 18432) * 1024,
+    "cgemm_splitk_kernel<2, 4>": (18463 * 2.0 + 18432) * 1024,
+}
+
 KERNEL_OF_STAGE = {"fft_a": "rfft2d_kernel", "fft_b": "rfft2d_kernel", "mm": "cgemm_freq_kernel",
                    "ifft": "irfft2d_kernel", "bias_grad": "bias_grad_dc_kernel"}
 
@@ -289,7 +298,7 @@ def main():
                 worst, worst_ms = (p, s, st), st["ms"]
     p, s, st = worst
     roofline = {"bound": st["bound"], "achieved": st["achieved"], "peak": st["peak"], "unit": st["unit"],
-                "frac": st["frac"], "traffic": None, "kernel": st["kernel"], "pass": p, "stage": s,
+                "frac": st["frac"], "traffic": MEASURED_TRAFFIC_MAIN.get(st["kernel"]), "kernel": st["kernel"], "pass": p, "stage": s,
                 "avg_launch_ms": st["ms"]}
 
     line = {

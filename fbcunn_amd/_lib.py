@@ -35,7 +35,8 @@ class PlanInfo(ctypes.Structure):
     _fields_ = [("fft_size", ctypes.c_int), ("n_freq", ctypes.c_int),
                 ("out_h", ctypes.c_int), ("out_w", ctypes.c_int),
                 ("input_freq_bytes", ctypes.c_size_t), ("weight_freq_bytes", ctypes.c_size_t),
-                ("output_freq_bytes", ctypes.c_size_t), ("scratch_bytes", ctypes.c_size_t)]
+                ("output_freq_bytes", ctypes.c_size_t), ("scratch_bytes", ctypes.c_size_t),
+                ("tiles_h", ctypes.c_int), ("tiles_w", ctypes.c_int)]
 
 
 _vp, _i, _f, _l = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
@@ -46,6 +47,8 @@ SIGNATURES = {
     "fbfc_last_error": (ctypes.c_char_p, []),
     "fbfc_plan_query": (_i, [ctypes.POINTER(ConvDesc), ctypes.POINTER(PlanInfo)]),
     "fbfc_plan_create": (_i, [ctypes.POINTER(ConvDesc), ctypes.POINTER(_vp)]),
+    "fbfc_plan_query_tiled": (_i, [ctypes.POINTER(ConvDesc), _i, _i, ctypes.POINTER(PlanInfo)]),
+    "fbfc_plan_create_tiled": (_i, [ctypes.POINTER(ConvDesc), _i, _i, ctypes.POINTER(_vp)]),
     "fbfc_plan_destroy": (_i, [_vp]),
     "fbfc_plan_get_info": (_i, [_vp, ctypes.POINTER(PlanInfo)]),
     "fbfc_update_output": (_i, [_vp, _vp, _vp, _vp, _vp, _vp]),
@@ -88,9 +91,13 @@ def check(rc):
     return rc
 
 
-def plan_query(**kw):
-    """Host-only planning: returns a PlanInfo or raises FbfcError (no GPU needed)."""
+def plan_query(tile_h=0, tile_w=0, **kw):
+    """Host-only planning: returns a PlanInfo or raises FbfcError (no GPU needed).
+    With tile sizes given, plans the tiled variant."""
     d = ConvDesc(**kw)
     info = PlanInfo()
-    check(lib().fbfc_plan_query(ctypes.byref(d), ctypes.byref(info)))
+    if tile_h or tile_w:
+        check(lib().fbfc_plan_query_tiled(ctypes.byref(d), tile_h, tile_w, ctypes.byref(info)))
+    else:
+        check(lib().fbfc_plan_query(ctypes.byref(d), ctypes.byref(info)))
     return info

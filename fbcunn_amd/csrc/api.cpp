@@ -31,6 +31,7 @@ int fail_hip(hipError_t e, const char *what)
 
 constexpr int kMinFft = 8;
 constexpr int kMaxFft = 128;
+constexpr int kMaxTileFft = 32;
 
 // fbcunn/SpatialConvolutionFFT.lua:875-882 (2^i, i = 1..10)
 int next_power_of_2(int v)
@@ -78,16 +79,82 @@ int plan_query(const fbfc_conv_desc *d, fbfc_plan_info *info)
     info->weight_freq_bytes = q * d->out_planes * d->in_planes * 8;
     info->output_freq_bytes = q * d->batch * d->out_planes * 8;
     info->scratch_bytes = fbfc::bias_grad_scratch_bytes(d->batch, d->out_planes);
+    info->tiles_h = 1;
+    info->tiles_w = 1;
     return FBFC_OK;
 }
 
+void set_geometry(fbfc_plan *p, int tile_h, int tile_w);
+
 bool fft_size_ok(int n) { return n == 8 || n == 16 || n == 32 || n == 64 || n == 128; }
 
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Tiled plans (fbcunn/SpatialConvolutionFFTTiled.lua:445-560, 618-672, 745-777): the tile is the
+// window that is transformed; consecutive windows are tile - kernel + 1 apart (overlap-save), so a
+// window yields that many finished rows / columns of the result.
+int plan_query_tiled(const fbfc_conv_desc *d, int tile_h, int tile_w, fbfc_plan_info *info)
+{
+    const int rc = plan_query(d, info);
+    // an image too large for one FFT is exactly what tiling is for
+    if (rc != FBFC_OK && rc != FBFC_ERR_UNSUPPORTED_SIZE) return rc;
+    const int out_h = d->in_h + 2 * d->pad_h - d->k_h + 1;
+    const int out_w = d->in_w + 2 * d->pad_w - d->k_w + 1;
+    char buf[160];
+    if (tile_h < 1 || tile_w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "both tile sizes must be specified");
+    if (tile_h < d->k_h || tile_w < d->k_w)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "Tiling cannot be smaller than kernel !");
+    if (tile_h > out_h || tile_w > out_w) {
+        std::snprintf(buf, sizeof buf, "Tile size too large (%dx%d) for output (%dx%d)", tile_h, tile_w, out_h,
+                      out_w);
+        return fail(FBFC_ERR_INVALID_ARGUMENT, buf);
+    }
+    int n = next_power_of_2(imax(tile_h, tile_w));
+    if (n < 0 || n > kMaxTileFft) {
+        std::snprintf(buf, sizeof buf, "tile FFT size not supported (tiles up to %d)", kMaxTileFft);
+        return fail(FBFC_ERR_UNSUPPORTED_SIZE, buf);
+    }
+    if (n < kMinFft) n = kMinFft;
+    const int step_h = tile_h - d->k_h + 1, step_w = tile_w - d->k_w + 1;
+    const size_t q = (size_t)n * (n / 2 + 1);
+    // output tiles (updateOutput, accGradParameters) and gradInput tiles (updateGradInput)
+    const size_t nt_out = (size_t)ceil_div(out_h, step_h) * ceil_div(out_w, step_w);
+    const size_t nt_in = (size_t)ceil_div(d->in_h, step_h) * ceil_div(d->in_w, step_w);
+    const size_t nt = nt_out > nt_in ? nt_out : nt_in;
+    info->fft_size = n;
+    info->n_freq = (int)q;
+    info->out_h = out_h;
+    info->out_w = out_w;
+    info->input_freq_bytes = q * d->batch * nt * d->in_planes * 8;
+    info->weight_freq_bytes = q * d->out_planes * d->in_planes * 8;
+    info->output_freq_bytes = q * d->batch * nt * d->out_planes * 8;
+    info->scratch_bytes = fbfc::bias_grad_scratch_bytes(d->batch, d->out_planes);
+    info->tiles_h = ceil_div(out_h, step_h);
+    info->tiles_w = ceil_div(out_w, step_w);
+    return FBFC_OK;
+}
+
 }  // namespace
+
+// What one pass transforms and contracts.  For an untiled plan the operands are whole planes and
+// vbatch is the batch; for a tiled plan they are windows and vbatch = batch * tiles.
+struct pass_geom {
+    int vbatch;
+    // forward-FFT operands that depend on tiling (the weight operand never does)
+    int a_h, a_w, a_pad_u, a_pad_l;   // input (fprop, accGrad) resp. gradOutput (bprop)
+    fbfc::Window a_win;
+    int g_h, g_w;                     // accGrad only: gradOutput
+    fbfc::Window g_win;
+    // inverse FFT
+    int r_h, r_w, r_pad_u, r_pad_l;
+    fbfc::Window r_win;
+};
 
 struct fbfc_plan {
     fbfc_conv_desc d;
     fbfc_plan_info info;
+    bool tiled;
+    pass_geom fprop, bprop, accgrad;
     int device;
     float *in_freq, *w_freq, *out_freq, *res_freq, *scratch;
     unsigned reuse;
@@ -153,6 +220,66 @@ struct StageTimer {
         }                                                      \
     } while (0)
 
+fbfc::Window make_window(int d1, int nty, int ntx, int step_y, int step_x, int off_y, int off_x, int img_h,
+                         int img_w)
+{
+    fbfc::Window w;
+    w.on = 1;
+    w.d1 = d1;
+    w.nt = nty * ntx;
+    w.ntx = ntx;
+    w.step_y = step_y;
+    w.step_x = step_x;
+    w.off_y = off_y;
+    w.off_x = off_x;
+    w.img_h = img_h;
+    w.img_w = img_w;
+    return w;
+}
+
+void set_geometry(fbfc_plan *p, int tile_h, int tile_w)
+{
+    const fbfc_conv_desc &d = p->d;
+    const int oh = p->info.out_h, ow = p->info.out_w;
+    pass_geom &f = p->fprop, &b = p->bprop, &a = p->accgrad;
+    if (!p->tiled) {
+        f.vbatch = b.vbatch = a.vbatch = d.batch;
+        f.a_h = d.in_h; f.a_w = d.in_w; f.a_pad_u = d.pad_h; f.a_pad_l = d.pad_w;
+        f.r_h = oh; f.r_w = ow;
+        b.a_h = oh; b.a_w = ow;
+        b.r_h = d.in_h; b.r_w = d.in_w; b.r_pad_u = d.pad_h; b.r_pad_l = d.pad_w;
+        a.a_h = d.in_h; a.a_w = d.in_w; a.a_pad_u = d.pad_h; a.a_pad_l = d.pad_w;
+        a.g_h = oh; a.g_w = ow;
+        a.r_h = d.k_h; a.r_w = d.k_w;
+        return;
+    }
+    const int sh = tile_h - d.k_h + 1, sw = tile_w - d.k_w + 1;
+    // updateOutput: output tiles sh x sw; input windows tile_h x tile_w whose corner is the tile's
+    // corner moved up-left by the padding (SpatialConvolutionFFTTiled.lua:521-537)
+    const int nty = ceil_div(oh, sh), ntx = ceil_div(ow, sw);
+    f.vbatch = d.batch * nty * ntx;
+    f.a_h = tile_h; f.a_w = tile_w;
+    f.a_win = make_window(d.in_planes, nty, ntx, sh, sw, -d.pad_h, -d.pad_w, d.in_h, d.in_w);
+    f.r_h = sh; f.r_w = sw;
+    f.r_win = make_window(d.out_planes, nty, ntx, sh, sw, 0, 0, oh, ow);
+    // updateGradInput: gradInput tiles sh x sw; gradOutput windows reach kernel - 1 further up-left,
+    // and the tile is read kernel - 1 rows / columns into the circular result (:638-658, :420-431)
+    const int mty = ceil_div(d.in_h, sh), mtx = ceil_div(d.in_w, sw);
+    b.vbatch = d.batch * mty * mtx;
+    b.a_h = tile_h; b.a_w = tile_w;
+    b.a_win = make_window(d.out_planes, mty, mtx, sh, sw, d.pad_h - (d.k_h - 1), d.pad_w - (d.k_w - 1), oh, ow);
+    b.r_h = sh; b.r_w = sw; b.r_pad_u = d.k_h - 1; b.r_pad_l = d.k_w - 1;
+    b.r_win = make_window(d.in_planes, mty, mtx, sh, sw, 0, 0, d.in_h, d.in_w);
+    // accGradParameters: gradOutput tiles sh x sw against the input windows of updateOutput; the sum
+    // over tiles joins the sum over the batch in the contraction (:758-777)
+    a.vbatch = f.vbatch;
+    a.a_h = tile_h; a.a_w = tile_w;
+    a.a_win = f.a_win;
+    a.g_h = sh; a.g_w = sw;
+    a.g_win = make_window(d.out_planes, nty, ntx, sh, sw, 0, 0, oh, ow);
+    a.r_h = d.k_h; a.r_w = d.k_w;
+}
+
 }  // namespace
 
 extern "C" {
@@ -166,18 +293,27 @@ int fbfc_plan_query(const fbfc_conv_desc *desc, fbfc_plan_info *info)
     return plan_query(desc, info);
 }
 
-int fbfc_plan_create(const fbfc_conv_desc *desc, fbfc_plan **out)
+int fbfc_plan_query_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan_info *info)
+{
+    if (desc == nullptr || info == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    return plan_query_tiled(desc, tile_h, tile_w, info);
+}
+
+static int plan_create(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **out)
 {
     if (out == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     *out = nullptr;
     fbfc_plan_info info;
-    const int rc = plan_query(desc, &info);
+    const bool tiled = tile_h > 0 || tile_w > 0;
+    const int rc = tiled ? fbfc_plan_query_tiled(desc, tile_h, tile_w, &info) : plan_query(desc, &info);
     if (rc != FBFC_OK) return rc;
     fbfc_plan *p = new (std::nothrow) fbfc_plan();
     if (p == nullptr) return fail(FBFC_ERR_OUT_OF_MEMORY, "host allocation failed");
     std::memset(p, 0, sizeof *p);
     p->d = *desc;
     p->info = info;
+    p->tiled = tiled;
+    set_geometry(p, tile_h, tile_w);
     hipError_t e = hipGetDevice(&p->device);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->in_freq), info.input_freq_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->w_freq), info.weight_freq_bytes);
@@ -192,6 +328,14 @@ int fbfc_plan_create(const fbfc_conv_desc *desc, fbfc_plan **out)
     }
     *out = p;
     return FBFC_OK;
+}
+
+int fbfc_plan_create(const fbfc_conv_desc *desc, fbfc_plan **out) { return plan_create(desc, 0, 0, out); }
+
+int fbfc_plan_create_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **out)
+{
+    if (tile_h < 1 || tile_w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "both tile sizes must be specified");
+    return plan_create(desc, tile_h, tile_w, out);
 }
 
 int fbfc_plan_destroy(fbfc_plan *p)
@@ -255,6 +399,13 @@ int fbfc_plan_stage_ms(const fbfc_plan *p, float *ms, int n)
     return FBFC_OK;
 }
 
+// the weight operand of updateOutput / updateGradInput: never windowed
+static fbfc::FwdArgs weight_args(const fbfc_plan *p, const float *weight)
+{
+    const fbfc_conv_desc &d = p->d;
+    return fbfc::FwdArgs{weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w, 0, 0, {}};
+}
+
 int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, const float *bias,
                        float *output, void *stream)
 {
@@ -262,17 +413,18 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
         return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const fbfc_conv_desc &d = p->d;
+    const pass_geom &g = p->fprop;
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
-    const fbfc::FwdArgs fin = {input, p->in_freq, (long)d.batch * d.in_planes, d.in_h, d.in_w, d.pad_h, d.pad_w};
-    const fbfc::FwdArgs fw = {weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w, 0, 0};
+    const fbfc::FwdArgs fin = {input, p->in_freq, (long)g.vbatch * d.in_planes, g.a_h, g.a_w, g.a_pad_u,
+                               g.a_pad_l, g.a_win};
+    const fbfc::FwdArgs fw = weight_args(p, weight);
     if (!p->timed) {  // both forward FFTs in one launch; timed plans keep them apart to time each
         FBFC_TRY(fbfc::launch_rfft2d_pair(N, fin, fw, s), "rfft2d(input, weight)");
     } else {
-        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fin.in, fin.out, fin.planes, fin.h, fin.w, fin.padU, fin.padL, s),
-                   "rfft2d(input)");
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fin, s), "rfft2d(input)");
         tm.done(FBFC_STAGE_FFT_A);
-        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fw.in, fw.out, fw.planes, fw.h, fw.w, 0, 0, s), "rfft2d(weight)");
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fw, s), "rfft2d(weight)");
         tm.done(FBFC_STAGE_FFT_B);
     }
     p->have_in = true;
@@ -280,11 +432,12 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     float *res = p->reuse ? p->res_freq : p->out_freq;
     if (!p->reuse) p->have_out = false;
     // O[b][f] = 1/N^2 sum_p I[b][p] conj(W[f][p])   (SpatialConvolutionFBFFT.lua:157-164)
-    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(0, p->in_freq, p->w_freq, res, Q, d.batch, d.out_planes,
+    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(0, p->in_freq, p->w_freq, res, Q, g.vbatch, d.out_planes,
                                      d.in_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(fprop)");
     tm.done(FBFC_STAGE_MM);
-    FBFC_STAGE(tm, fbfc::launch_irfft2d(N, res, output, (long)d.batch * d.out_planes, p->info.out_h,
-                                  p->info.out_w, 0, 0, bias, d.out_planes, s), "irfft2d(output)");
+    const fbfc::InvArgs inv = {res, output, (long)g.vbatch * d.out_planes, g.r_h, g.r_w, g.r_pad_u, g.r_pad_l,
+                               bias, d.out_planes, g.r_win, nullptr, nullptr, 0.0f, 0, 0};
+    FBFC_STAGE(tm, fbfc::launch_irfft2d_args(N, inv, s), "irfft2d(output)");
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();
 }
@@ -296,33 +449,35 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
         return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const fbfc_conv_desc &d = p->d;
+    const pass_geom &g = p->bprop;
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
-    const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)d.batch * d.out_planes, p->info.out_h,
-                               p->info.out_w, 0, 0};
-    const fbfc::FwdArgs fw = {weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w, 0, 0};
+    const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)g.vbatch * d.out_planes, g.a_h, g.a_w,
+                               g.a_pad_u, g.a_pad_l, g.a_win};
+    const fbfc::FwdArgs fw = weight_args(p, weight);
     const bool need_w = !((p->reuse & FBFC_REUSE_WEIGHT) && p->have_w);
     if (!p->timed && need_w) {
         FBFC_TRY(fbfc::launch_rfft2d_pair(N, fgo, fw, s), "rfft2d(gradOutput, weight)");
     } else {
-        FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fgo.in, fgo.out, fgo.planes, fgo.h, fgo.w, 0, 0, s),
-                   "rfft2d(gradOutput)");
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fgo, s), "rfft2d(gradOutput)");
         tm.done(FBFC_STAGE_FFT_A);
         if (need_w) {
-            FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fw.in, fw.out, fw.planes, fw.h, fw.w, 0, 0, s), "rfft2d(weight)");
+            FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fw, s), "rfft2d(weight)");
             tm.done(FBFC_STAGE_FFT_B);
         }
     }
-    p->have_out = true;
+    // a tiled updateGradInput transforms other windows of gradOutput than accGradParameters does
+    p->have_out = !p->tiled;
     p->have_w = true;
     float *res = p->reuse ? p->res_freq : p->in_freq;
     if (!p->reuse) p->have_in = false;
     // GI[b][p] = 1/N^2 sum_f GO[b][f] W[f][p]   (SpatialConvolutionFBFFT.lua:244-251)
-    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(1, p->out_freq, p->w_freq, res, Q, d.batch, d.in_planes,
+    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(1, p->out_freq, p->w_freq, res, Q, g.vbatch, d.in_planes,
                                      d.out_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(bprop)");
     tm.done(FBFC_STAGE_MM);
-    FBFC_STAGE(tm, fbfc::launch_irfft2d(N, res, grad_input, (long)d.batch * d.in_planes, d.in_h, d.in_w,
-                                  d.pad_h, d.pad_w, nullptr, 1, s), "irfft2d(gradInput)");
+    const fbfc::InvArgs inv = {res, grad_input, (long)g.vbatch * d.in_planes, g.r_h, g.r_w, g.r_pad_u,
+                               g.r_pad_l, nullptr, 1, g.r_win, nullptr, nullptr, 0.0f, 0, 0};
+    FBFC_STAGE(tm, fbfc::launch_irfft2d_args(N, inv, s), "irfft2d(gradInput)");
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();
 }
@@ -334,24 +489,24 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
         return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const fbfc_conv_desc &d = p->d;
+    const pass_geom &g = p->accgrad;
     const int N = p->info.fft_size, Q = p->info.n_freq;
     StageTimer tm(p, s);
-    const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)d.batch * d.out_planes, p->info.out_h,
-                               p->info.out_w, 0, 0};
-    const fbfc::FwdArgs fin = {input, p->in_freq, (long)d.batch * d.in_planes, d.in_h, d.in_w, d.pad_h, d.pad_w};
+    const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)g.vbatch * d.out_planes, g.g_h, g.g_w, 0, 0,
+                               g.g_win};
+    const fbfc::FwdArgs fin = {input, p->in_freq, (long)g.vbatch * d.in_planes, g.a_h, g.a_w, g.a_pad_u,
+                               g.a_pad_l, g.a_win};
     const bool need_go = !((p->reuse & FBFC_REUSE_OUTPUT) && p->have_out);
     const bool need_in = !((p->reuse & FBFC_REUSE_INPUT) && p->have_in);
     if (!p->timed && need_go && need_in) {
         FBFC_TRY(fbfc::launch_rfft2d_pair(N, fgo, fin, s), "rfft2d(gradOutput, input)");
     } else {
         if (need_go) {
-            FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fgo.in, fgo.out, fgo.planes, fgo.h, fgo.w, 0, 0, s),
-                       "rfft2d(gradOutput)");
+            FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fgo, s), "rfft2d(gradOutput)");
             tm.done(FBFC_STAGE_FFT_A);
         }
         if (need_in) {
-            FBFC_STAGE(tm, fbfc::launch_rfft2d(N, fin.in, fin.out, fin.planes, fin.h, fin.w, fin.padU, fin.padL, s),
-                       "rfft2d(input)");
+            FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fin, s), "rfft2d(input)");
             tm.done(FBFC_STAGE_FFT_B);
         }
     }
@@ -360,7 +515,7 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     // gradBias[f] = scale * sum_b DC(gradOutput[b][f]) is read off the spectrum just computed:
     // its own launch when timed, otherwise a few extra workgroups of the inverse-FFT launch.
     if (grad_bias != nullptr && p->timed) {
-        FBFC_STAGE(tm, fbfc::launch_bias_grad_dc(p->out_freq, grad_bias, scale, d.batch, d.out_planes, s),
+        FBFC_STAGE(tm, fbfc::launch_bias_grad_dc(p->out_freq, grad_bias, scale, g.vbatch, d.out_planes, s),
                    "bias grad");
         tm.done(FBFC_STAGE_BIAS_GRAD);
     }
@@ -368,15 +523,19 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     if (!p->reuse) p->have_w = false;
     // GW[f][p] = scale/N^2 sum_b conj(GO[b][f]) I[b][p]   (SpatialConvolutionFBFFT.lua:337-344)
     FBFC_STAGE(tm, fbfc::launch_cgemm_freq(2, p->out_freq, p->in_freq, res, Q, d.out_planes, d.in_planes,
-                                     d.batch, scale / ((float)N * (float)N), 0, s), "cgemm(accGrad)");
+                                     g.vbatch, scale / ((float)N * (float)N), 0, s), "cgemm(accGrad)");
     tm.done(FBFC_STAGE_MM);
+    fbfc::InvArgs inv = {res, grad_weight, (long)d.out_planes * d.in_planes, g.r_h, g.r_w, 0, 0, nullptr, 1, {},
+                         nullptr, nullptr, 0.0f, 0, 0};
     if (grad_bias != nullptr && !p->timed) {
-        FBFC_TRY(fbfc::launch_irfft2d_bias_grad(N, res, grad_weight, (long)d.out_planes * d.in_planes, d.k_h,
-                                                d.k_w, p->out_freq, grad_bias, scale, d.batch,
-                                                d.out_planes, s), "irfft2d(gradWeight) + bias grad");
+        inv.go_freq = p->out_freq;
+        inv.grad_bias = grad_bias;
+        inv.scale = scale;
+        inv.batch = g.vbatch;
+        inv.out_planes = d.out_planes;
+        FBFC_TRY(fbfc::launch_irfft2d_args(N, inv, s), "irfft2d(gradWeight) + bias grad");
     } else {
-        FBFC_STAGE(tm, fbfc::launch_irfft2d(N, res, grad_weight, (long)d.out_planes * d.in_planes, d.k_h,
-                                            d.k_w, 0, 0, nullptr, 1, s), "irfft2d(gradWeight)");
+        FBFC_STAGE(tm, fbfc::launch_irfft2d_args(N, inv, s), "irfft2d(gradWeight)");
     }
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();

@@ -135,6 +135,56 @@ __device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int 
 }
 
 // ---------------------------------------------------------------------------------
+// Windows (tiled convolution).  A windowed operand is a (d0, d1, img_h, img_w) tensor seen as
+// d0 * nt * d1 "virtual planes" of h x w: virtual plane v = (b * nt + tile) * d1 + c is the window
+// of plane (b, c) whose corner is (ty * step_y + off_y, tx * step_x + off_x), tile = ty * ntx + tx.
+// Reads outside the image give zero, writes outside it are dropped.  The staging area keeps the
+// same canvas-row layout (padL = 0 on the way in), so the transforms themselves do not change.
+// ---------------------------------------------------------------------------------
+// per virtual plane of the workgroup: element offset of its image plane (lo, hi) and window corner
+template <int N>
+__device__ __forceinline__ void build_window_table(int4 *tbl, const Window &win, long x0, long planes, int tid)
+{
+    if (tid < FftShape<N>::T) {
+        long v = x0 + tid;
+        if (v >= planes) v = planes - 1;
+        const long vb = v / win.d1;
+        const int c = (int)(v - vb * win.d1);
+        const long b = vb / win.nt;
+        const int tile = (int)(vb - b * win.nt);
+        const int ty = tile / win.ntx, tx = tile - ty * win.ntx;
+        const long off = (b * win.d1 + c) * ((long)win.img_h * win.img_w);
+        tbl[tid] = make_int4((int)(unsigned)(off & 0xffffffffL), (int)(off >> 32),
+                             ty * win.step_y + win.off_y, tx * win.step_x + win.off_x);
+    }
+}
+
+// nrows = nph * h canvas rows of the planes [first, first + nph) of the workgroup
+template <int N, bool TO_LDS>
+__device__ __forceinline__ void copy_windows(float *smem, float *g, const int4 *tbl, int first, int nph,
+                                             int h, int w, int padL, const Window &win, int tid)
+{
+    constexpr int LDR = Canvas<N>::LDR;
+    const int total = nph * h * N;
+    const int magic = (1 << 20) / h + 1;  // rr / h for rr < 512 <= T * h
+    for (int e = tid; e < total; e += 256) {
+        const int c = e % N, rr = e / N;
+        const int tl = (rr * magic) >> 20;
+        const int r = rr - tl * h;
+        const int4 q = tbl[first + tl];
+        const int y = q.z + r, x = q.w + c;
+        const bool ok = (c < w) && ((unsigned)y < (unsigned)win.img_h) && ((unsigned)x < (unsigned)win.img_w);
+        float *gp = g + ((((long)q.y) << 32) | (long)(unsigned)q.x) + (long)y * win.img_w + x;
+        float *sp = smem + rr * LDR + padL + c;
+        if (TO_LDS) {
+            *sp = ok ? *gp : 0.0f;
+        } else if (ok) {
+            *gp = *sp;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // forward: real (planes,h,w) -> freq [N*(N/2+1)][planes] complex
 // ---------------------------------------------------------------------------------
 // One launch can transform two tensors of the same FFT size (the two forward FFTs of a pass):
@@ -144,9 +194,11 @@ struct FwdJob {
     float2 *out;
     long planes;
     int h, w, padU, padL, vec4;
+    int tbl_off;  // windowed operand: float offset of the window table in LDS
+    Window win;
 };
 
-template <int N>
+template <int N, bool WIN>
 __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(FwdJob job0, FwdJob job1,
                                                                       unsigned blocks0)
 {
@@ -165,6 +217,11 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
+    [[maybe_unused]] const Window &win = second ? job1.win : job0.win;
+    [[maybe_unused]] int4 *tbl = reinterpret_cast<int4 *>(smem + (second ? job1.tbl_off : job0.tbl_off));
+    if constexpr (WIN) {
+        if (win.on) build_window_table<N>(tbl, win, x0, planes, tid);
+    }
     const int y_lo = padU & ~1;                       // first canvas row that can be non-zero (even)
     const int y_hi = (padU + h + 1) & ~1;             // one past the last, rounded up to even
 
@@ -187,8 +244,16 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
         int nph = np - hs * S::TP;
         nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
         if (hs > 0) __syncthreads();  // previous round fully read
-        zero_canvas_margins<N>(smem, nph * h, w, padL, zrow, tid);
-        copy_canvas<N, true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
+        bool windowed = false;
+        if constexpr (WIN) windowed = win.on != 0;
+        if (windowed) {
+            if (hs == 0) __syncthreads();  // window table complete
+            zero_canvas_margins<N>(smem, 0, w, 0, zrow, tid);  // the all-zero row only
+            copy_windows<N, true>(smem, const_cast<float *>(in), tbl, hs * S::TP, nph, h, w, 0, win, tid);
+        } else {
+            zero_canvas_margins<N>(smem, nph * h, w, padL, zrow, tid);
+            copy_canvas<N, true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
+        }
         __syncthreads();
         if (row_active && (t / S::TP) == hs) {
             const int tl = t - hs * S::TP;
@@ -300,13 +365,13 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
 // inverse: freq [N*(N/2+1)][planes] complex -> real (planes,h,w), unnormalised,
 // real[r][s] = y[r+padU][s+padL] (+ bias[plane % bias_period])
 // ---------------------------------------------------------------------------------
-template <int N>
+template <int N, bool WIN>
 __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void irfft2d_kernel(const float2 *__restrict__ in,
                                                       float *__restrict__ out, long planes,
                                                       int h, int w, int padU, int padL,
                                                       const float *__restrict__ bias,
                                                       int bias_period, int vec4, BiasGradJob bgrad,
-                                                      unsigned bgrad_blocks)
+                                                      unsigned bgrad_blocks, Window win, int tbl_off)
 {
     using S = FftShape<N>;
     constexpr int T = S::T;
@@ -322,6 +387,11 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void irfft2d_kernel(co
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
+    [[maybe_unused]] int4 *tbl = reinterpret_cast<int4 *>(smem + tbl_off);
+    if constexpr (WIN) {
+        // read again only after the barriers of the passes below
+        if (win.on) build_window_table<N>(tbl, win, x0, planes, tid);
+    }
     const int y_lo = padU & ~1;                       // canvas rows the crop needs
     const int y_hi = (padU + h + 1) & ~1;
 
@@ -433,7 +503,12 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void irfft2d_kernel(co
             }
         }
         __syncthreads();
-        copy_canvas<N, false>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
+        bool windowed = false;
+        if constexpr (WIN) windowed = win.on != 0;
+        if (windowed)
+            copy_windows<N, false>(smem, out, tbl, hs * S::TP, nph, h, w, padL, win, tid);
+        else
+            copy_canvas<N, false>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
     });
 }
 
@@ -462,25 +537,34 @@ static long fwd_blocks(long planes)
 }
 
 template <int N>
-static FwdJob make_job(const float *in, float *out, long planes, int h, int w, int padU, int padL)
+static FwdJob make_job(const FwdArgs &a)
 {
     using S = FftShape<N>;
     FwdJob j;
-    j.in = in;
-    j.out = reinterpret_cast<float2 *>(out);
-    j.planes = planes;
-    j.h = h; j.w = w; j.padU = padU; j.padL = padL;
-    j.vec4 = ((reinterpret_cast<uintptr_t>(in) & 15) == 0) && (((long)S::T * h * w) % 4 == 0);
+    j.in = a.in;
+    j.out = reinterpret_cast<float2 *>(a.out);
+    j.planes = a.planes;
+    j.h = a.h; j.w = a.w; j.padU = a.padU; j.padL = a.padL;
+    j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::T * a.h * a.w) % 4 == 0);
+    j.tbl_off = 0;
+    j.win = a.win;
     return j;
 }
 
+static bool window_ok(const Window &w, long planes, int h, int ww)
+{
+    if (!w.on) return true;
+    return w.d1 > 0 && w.nt > 0 && w.ntx > 0 && w.nt % w.ntx == 0 && w.step_y > 0 && w.step_x > 0 &&
+           w.img_h > 0 && w.img_w > 0 && h > 0 && ww > 0 && planes % ((long)w.nt * w.d1) == 0;
+}
+
 // second == nullptr: one tensor only
-template <int N>
+template <int N, bool WIN>
 static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
 {
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rfft2d_kernel<N>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rfft2d_kernel<N, WIN>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         attr_done = true;
@@ -488,42 +572,48 @@ static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_
     size_t lds = fft_lds_bytes<N>(a.h, a.w, a.padU, false);
     const long blocks0 = fwd_blocks<N>(a.planes);
     long blocks = blocks0;
-    const FwdJob j0 = make_job<N>(a.in, a.out, a.planes, a.h, a.w, a.padU, a.padL);
+    FwdJob j0 = make_job<N>(a);
     FwdJob j1 = j0;
     if (second != nullptr) {
         const size_t lds1 = fft_lds_bytes<N>(second->h, second->w, second->padU, false);
         if (lds1 > lds) lds = lds1;
         blocks += fwd_blocks<N>(second->planes);
-        j1 = make_job<N>(second->in, second->out, second->planes, second->h, second->w, second->padU,
-                         second->padL);
+        j1 = make_job<N>(*second);
+    }
+    if (WIN) {  // the window table sits behind the tile / staging area
+        j0.tbl_off = j1.tbl_off = (int)(lds / sizeof(float));
+        lds += FftShape<N>::T * sizeof(int4);
     }
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(rfft2d_kernel<N>, dim3((unsigned)blocks), dim3(256), lds, s, j0, j1,
+    hipLaunchKernelGGL((rfft2d_kernel<N, WIN>), dim3((unsigned)blocks), dim3(256), lds, s, j0, j1,
                        (unsigned)blocks0);
     return hipGetLastError();
 }
 
-template <int N>
-static hipError_t launch_inv(const float *in, float *out, long planes, int h, int w, int padU,
-                             int padL, const float *bias, int bias_period, const BiasGradJob &bgrad,
-                             hipStream_t s)
+template <int N, bool WIN>
+static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
 {
     using S = FftShape<N>;
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&irfft2d_kernel<N>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&irfft2d_kernel<N, WIN>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    const size_t lds = fft_lds_bytes<N>(h, w, padU, true);
-    long blocks = (planes + S::T - 1) / S::T;
+    size_t lds = fft_lds_bytes<N>(a.h, a.w, a.padU, true);
+    const int tbl_off = (int)(lds / sizeof(float));
+    if (WIN) lds += S::T * sizeof(int4);
+    long blocks = (a.planes + S::T - 1) / S::T;
     if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
-    const int vec4 = ((reinterpret_cast<uintptr_t>(out) & 15) == 0) && (((long)S::T * h * w) % 4 == 0);
+    const int vec4 = ((reinterpret_cast<uintptr_t>(a.out) & 15) == 0) && (((long)S::T * a.h * a.w) % 4 == 0);
+    const BiasGradJob bgrad = {reinterpret_cast<const float2 *>(a.go_freq), a.grad_bias, a.scale, a.batch,
+                               a.out_planes};
     const unsigned bblocks = (bgrad.dc != nullptr) ? bias_grad_dc_blocks(bgrad.planes) : 0u;
-    hipLaunchKernelGGL(irfft2d_kernel<N>, dim3((unsigned)blocks + bblocks), dim3(256), lds, s,
-                       reinterpret_cast<const float2 *>(in), out, planes, h, w, padU, padL, bias,
-                       bias_period > 0 ? bias_period : 1, vec4, bgrad, bblocks);
+    if (blocks + bblocks > 0x7fffffffL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((irfft2d_kernel<N, WIN>), dim3((unsigned)blocks + bblocks), dim3(256), lds, s,
+                       reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL,
+                       a.bias, a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks, a.win, tbl_off);
     return hipGetLastError();
 }
 
@@ -533,12 +623,22 @@ static bool planes_ok(int N, long planes) { return planes > 0 && (long)(N / 2 + 
 static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s)
 {
     if (!planes_ok(N, a.planes) || (b != nullptr && !planes_ok(N, b->planes))) return hipErrorInvalidValue;
+    if (!window_ok(a.win, a.planes, a.h, a.w) || (b != nullptr && !window_ok(b->win, b->planes, b->h, b->w)))
+        return hipErrorInvalidValue;
+    if (a.win.on || (b != nullptr && b->win.on)) {
+        switch (N) {
+            case 8: return launch_fwd<8, true>(a, b, s);
+            case 16: return launch_fwd<16, true>(a, b, s);
+            case 32: return launch_fwd<32, true>(a, b, s);
+            default: return hipErrorInvalidValue;
+        }
+    }
     switch (N) {
-        case 8: return launch_fwd<8>(a, b, s);
-        case 16: return launch_fwd<16>(a, b, s);
-        case 32: return launch_fwd<32>(a, b, s);
-        case 64: return launch_fwd<64>(a, b, s);
-        case 128: return launch_fwd<128>(a, b, s);
+        case 8: return launch_fwd<8, false>(a, b, s);
+        case 16: return launch_fwd<16, false>(a, b, s);
+        case 32: return launch_fwd<32, false>(a, b, s);
+        case 64: return launch_fwd<64, false>(a, b, s);
+        case 128: return launch_fwd<128, false>(a, b, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -546,26 +646,34 @@ static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStr
 hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                          int padL, hipStream_t s)
 {
-    const FwdArgs a = {in, out, planes, h, w, padU, padL};
+    const FwdArgs a = {in, out, planes, h, w, padU, padL, {}};
     return dispatch_fwd(N, a, nullptr, s);
 }
+
+hipError_t launch_rfft2d_one(int N, const FwdArgs &a, hipStream_t s) { return dispatch_fwd(N, a, nullptr, s); }
 
 hipError_t launch_rfft2d_pair(int N, const FwdArgs &a, const FwdArgs &b, hipStream_t s)
 {
     return dispatch_fwd(N, a, &b, s);
 }
 
-static hipError_t dispatch_inv(int N, const float *in, float *out, long planes, int h, int w, int padU,
-                               int padL, const float *bias, int bias_period, const BiasGradJob &bgrad,
-                               hipStream_t s)
+hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s)
 {
-    if (!planes_ok(N, planes)) return hipErrorInvalidValue;
+    if (!planes_ok(N, a.planes) || !window_ok(a.win, a.planes, a.h, a.w)) return hipErrorInvalidValue;
+    if (a.win.on) {
+        switch (N) {
+            case 8: return launch_inv<8, true>(a, s);
+            case 16: return launch_inv<16, true>(a, s);
+            case 32: return launch_inv<32, true>(a, s);
+            default: return hipErrorInvalidValue;
+        }
+    }
     switch (N) {
-        case 8: return launch_inv<8>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
-        case 16: return launch_inv<16>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
-        case 32: return launch_inv<32>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
-        case 64: return launch_inv<64>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
-        case 128: return launch_inv<128>(in, out, planes, h, w, padU, padL, bias, bias_period, bgrad, s);
+        case 8: return launch_inv<8, false>(a, s);
+        case 16: return launch_inv<16, false>(a, s);
+        case 32: return launch_inv<32, false>(a, s);
+        case 64: return launch_inv<64, false>(a, s);
+        case 128: return launch_inv<128, false>(a, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -573,16 +681,16 @@ static hipError_t dispatch_inv(int N, const float *in, float *out, long planes, 
 hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                           int padL, const float *bias, int bias_period, hipStream_t s)
 {
-    const BiasGradJob none = {nullptr, nullptr, 0.0f, 0, 0};
-    return dispatch_inv(N, in, out, planes, h, w, padU, padL, bias, bias_period, none, s);
+    const InvArgs a = {in, out, planes, h, w, padU, padL, bias, bias_period, {}, nullptr, nullptr, 0.0f, 0, 0};
+    return launch_irfft2d_args(N, a, s);
 }
 
 hipError_t launch_irfft2d_bias_grad(int N, const float *in, float *out, long planes, int h, int w,
                                     const float *go_freq, float *grad_bias, float scale, int batch,
                                     int out_planes, hipStream_t s)
 {
-    const BiasGradJob job = {reinterpret_cast<const float2 *>(go_freq), grad_bias, scale, batch, out_planes};
-    return dispatch_inv(N, in, out, planes, h, w, 0, 0, nullptr, 1, job, s);
+    const InvArgs a = {in, out, planes, h, w, 0, 0, nullptr, 1, {}, go_freq, grad_bias, scale, batch, out_planes};
+    return launch_irfft2d_args(N, a, s);
 }
 
 }  // namespace fbfc

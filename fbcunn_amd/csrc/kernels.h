@@ -9,14 +9,24 @@ namespace fbfc {
 // N in {8,16,32,64,128}; any other value returns hipErrorInvalidValue.
 hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                          int padL, hipStream_t s);
+// A (d0, d1, img_h, img_w) tensor seen through windows (tiled convolution): virtual plane
+// v = (b * nt + tile) * d1 + c is the h x w window of plane (b, c) with corner
+// (ty * step_y + off_y, tx * step_x + off_x), tile = ty * ntx + tx.  Outside the image reads give
+// zero and writes are dropped.  on = 0: ordinary contiguous planes.  Windows need N <= 32.
+struct Window {
+    int on;
+    int d1, nt, ntx, step_y, step_x, off_y, off_x, img_h, img_w;
+};
 // Two forward transforms of the same size in one launch (the two FFTs of a pass).
 struct FwdArgs {
     const float *in;
     float *out;
-    long planes;
+    long planes;  // virtual planes when windowed
     int h, w, padU, padL;
+    Window win;
 };
 hipError_t launch_rfft2d_pair(int N, const FwdArgs &a, const FwdArgs &b, hipStream_t s);
+hipError_t launch_rfft2d_one(int N, const FwdArgs &a, hipStream_t s);
 hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                           int padL, const float *bias, int bias_period, hipStream_t s);
 
@@ -25,6 +35,23 @@ hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h
 hipError_t launch_irfft2d_bias_grad(int N, const float *in, float *out, long planes, int h, int w,
                                     const float *go_freq, float *grad_bias, float scale, int batch,
                                     int out_planes, hipStream_t s);
+
+// General form of the inverse: optional bias add, optional windowed store, optional bias-gradient job
+// (go_freq != nullptr: grad_bias[f] = scale * sum_{b < batch} Re go_freq[0][b][f]).
+struct InvArgs {
+    const float *in;
+    float *out;
+    long planes;
+    int h, w, padU, padL;
+    const float *bias;
+    int bias_period;
+    Window win;
+    const float *go_freq;
+    float *grad_bias;
+    float scale;
+    int batch, out_planes;
+};
+hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s);
 
 // cgemm_kernels.hip ------------------------------------------------------------
 // mode 0: C[m][n] (+)= alpha * sum_k A[m][k] * conj(B[n][k])   A (m x k), B (n x k)

@@ -16,7 +16,8 @@ from . import _lib
 from ._lib import ConvDesc, FbfcError, PlanInfo, check, lib
 
 __all__ = ["SpatialConvolutionFFT", "SpatialConvolutionFBFFT", "SpatialConvolutionFBFFTGemm",
-           "FFTWrapper", "transposeMM", "updateOutputBias", "accGradParametersBias", "FbfcError"]
+           "SpatialConvolutionFFTTiled", "SpatialConvolutionFFTTiledSync", "SpatialConvolutionFFTTiledAsync",
+           "SpatialConvolutionFFTTiledIterated", "FFTWrapper", "transposeMM", "updateOutputBias", "accGradParametersBias", "FbfcError"]
 
 
 def _ptr(t):
@@ -41,9 +42,12 @@ def _check_tensor(t, name, ndim=None):
 class _Plan:
     """RAII holder of one fbfc_plan."""
 
-    def __init__(self, desc):
+    def __init__(self, desc, tile=None):
         self.handle = ctypes.c_void_p(0)
-        check(lib().fbfc_plan_create(ctypes.byref(desc), ctypes.byref(self.handle)))
+        if tile is None:
+            check(lib().fbfc_plan_create(ctypes.byref(desc), ctypes.byref(self.handle)))
+        else:
+            check(lib().fbfc_plan_create_tiled(ctypes.byref(desc), tile[0], tile[1], ctypes.byref(self.handle)))
         self.info = PlanInfo()
         check(lib().fbfc_plan_get_info(self.handle, ctypes.byref(self.info)))
 
@@ -131,12 +135,16 @@ class SpatialConvolutionFFT:
         if plan is None:
             desc = ConvDesc(batch, self.nInputPlane, self.nOutputPlane, in_h, in_w, self.kH, self.kW,
                             self.dH, self.dW, self.padUp, self.padLeft)
-            plan = _Plan(desc)
+            plan = _Plan(desc, self._tile())
             if self._reuse_bits:
                 check(lib().fbfc_plan_set_reuse(plan.handle, self._reuse_bits))
             self._plans[key] = plan
         check(lib().fbfc_plan_set_timed(plan.handle, int(self.timed)))  # reps per stage, 0 = off
         return plan
+
+    def _tile(self):
+        """(tileSizeH, tileSizeW) of a tiled module, None otherwise."""
+        return None
 
     def _check_input(self, input):
         _check_tensor(input, "input", 4)
@@ -214,6 +222,39 @@ class SpatialConvolutionFBFFTGemm(SpatialConvolutionFFT):
     done (explicit transposes + cuBLAS Cgemm); here both modules share the one
     frequency-major MFMA contraction, which is the layout that variant builds."""
     fftImplementation = "fbfft"
+
+
+class SpatialConvolutionFFTTiled(SpatialConvolutionFBFFT):
+    """nn.SpatialConvolutionFFTTiled (fbcunn/SpatialConvolutionFFTTiled.lua:260-330): the image is
+    convolved window by window with FFTs of the tile size (default 16) instead of one FFT that
+    covers the whole image.  Constructor arguments in the reference's order."""
+
+    def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padLeft=0, padUp=0,
+                 tileSizeW=None, tileSizeH=None, memoryReusePolicy=None, numCudaStreams=None, device="cuda"):
+        for v in (tileSizeW, tileSizeH):
+            if v is not None and not isinstance(v, int):
+                raise TypeError("tile sizes must be numbers")
+        self.tileSizeH = tileSizeH or 16
+        self.tileSizeW = tileSizeW or 16
+        super().__init__(nInputPlane, nOutputPlane, kW, kH, dW, dH, padLeft, padUp, memoryReusePolicy,
+                         numCudaStreams, device)
+
+    def _tile(self):
+        return (self.tileSizeH, self.tileSizeW)
+
+
+class SpatialConvolutionFFTTiledSync(SpatialConvolutionFFTTiled):
+    """nn.SpatialConvolutionFFTTiledSync (fbcunn/SpatialConvolutionFFTTiledSync.lua): in the
+    reference one tile after the other on one stream; here all tiles go through each stage in a
+    single launch, so the Sync / Async / Iterated variants are one implementation."""
+
+
+class SpatialConvolutionFFTTiledAsync(SpatialConvolutionFFTTiled):
+    """nn.SpatialConvolutionFFTTiledAsync (fbcunn/SpatialConvolutionFFTTiledAsync.lua)."""
+
+
+class SpatialConvolutionFFTTiledIterated(SpatialConvolutionFFTTiled):
+    """nn.SpatialConvolutionFFTTiledIterated (fbcunn/SpatialConvolutionFFTTiledIterated.lua)."""
 
 
 class FFTWrapper:

@@ -59,6 +59,7 @@ typedef struct {
     size_t weight_freq_bytes;  /* Q * F * P * 8 */
     size_t output_freq_bytes;  /* Q * B * F * 8 */
     size_t scratch_bytes;      /* what fbfc_acc_grad_parameters_bias needs for this shape */
+    int tiles_h, tiles_w;      /* output tiles per image (1 x 1 for an untiled plan) */
 } fbfc_plan_info;
 
 typedef struct fbfc_plan fbfc_plan;
@@ -84,6 +85,20 @@ int fbfc_plan_query(const fbfc_conv_desc *desc, fbfc_plan_info *info);
 int fbfc_plan_create(const fbfc_conv_desc *desc, fbfc_plan **plan);
 int fbfc_plan_destroy(fbfc_plan *plan);
 int fbfc_plan_get_info(const fbfc_plan *plan, fbfc_plan_info *info);
+
+/* Tiled plans: nn.SpatialConvolutionFFTTiled and its Sync / Async / Iterated instantiations
+ * (fbcunn/SpatialConvolutionFFTTiled.lua:260-330 constructor, :445-560, :618-672, :745-777 tilings).
+ * The image is cut into windows of tile_h x tile_w (the reference's tileSizeH / tileSizeW, default
+ * 16) that are tile - kernel + 1 apart; each window is transformed with an FFT of the next power
+ * of two (8, 16 or 32), so images far larger than one FFT are convolved with small transforms.
+ * Results equal those of an untiled plan.  The passes are the same three entry points below; a
+ * tiled plan's buffers hold batch * tiles planes.  Errors follow the reference: tile smaller than
+ * the kernel ("Tiling cannot be smaller than kernel !"), tile larger than the output ("Tile size
+ * too large ..."); tiles above 32 are FBFC_ERR_UNSUPPORTED_SIZE.  With a reuse policy set, the
+ * spectrum of gradOutput is never reused (updateGradInput and accGradParameters window it
+ * differently). */
+int fbfc_plan_query_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan_info *info);
+int fbfc_plan_create_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **plan);
 
 /* Replaces SpatialConvolutionFBFFT:updateOutputFFTImpl
  * (fbcunn/SpatialConvolutionFBFFT.lua:102-183):

@@ -73,3 +73,43 @@ def test_plan_rejections(kw, code, text):
 def test_scratch_size_query():
     assert _lib.lib().fbfc_bias_grad_scratch_bytes(128, 64) >= 64 * 4
     assert _lib.lib().fbfc_bias_grad_scratch_bytes(0, 64) == 0
+
+
+# Tiled planning (fbcunn/SpatialConvolutionFFTTiled.lua:521-537): windows of the tile size,
+# tile - kernel + 1 apart; the FFT is the next power of two of the tile.
+@pytest.mark.parametrize("kw,tile,n,tiles", [
+    (dict(in_h=112, in_w=112), (32, 32), 32, (4, 4)),          # o = 112, step 30
+    (dict(in_h=224, in_w=224), (32, 32), 32, (8, 8)),          # o = 224, step 30
+    (dict(in_h=56, in_w=56), (16, 16), 16, (4, 4)),            # o = 56, step 14
+    (dict(in_h=45, in_w=52), (10, 14), 16, (6, 5)),            # steps 8 and 12
+    (dict(in_h=20, in_w=20, k_h=5, k_w=5, pad_h=0, pad_w=0), (8, 8), 8, (4, 4)),   # o = 16, step 4
+])
+def test_tiled_plan_sizes(kw, tile, n, tiles):
+    info = _q(**dict(kw, tile_h=tile[0], tile_w=tile[1]))
+    assert info.fft_size == n and (info.tiles_h, info.tiles_w) == tiles
+    q = n * (n // 2 + 1)
+    assert info.n_freq == q
+    # buffers hold batch * tiles planes (tiles of the output, or of gradInput if those are more)
+    assert info.output_freq_bytes >= q * 2 * tiles[0] * tiles[1] * 4 * 8
+    assert _q(**kw).tiles_h == 1 if max(kw["in_h"], kw["in_w"]) <= 126 else True
+
+
+@pytest.mark.parametrize("kw,tile,code,text", [
+    (dict(in_h=20, in_w=20, k_h=5, k_w=5, pad_h=0, pad_w=0), (4, 4), _lib.ERR_INVALID_ARGUMENT,
+     "Tiling cannot be smaller than kernel"),
+    (dict(in_h=20, in_w=20), (32, 32), _lib.ERR_INVALID_ARGUMENT, "Tile size too large (32x32) for output (20x20)"),
+    (dict(in_h=100, in_w=100), (64, 64), _lib.ERR_UNSUPPORTED_SIZE, "tile FFT size"),
+    (dict(in_h=100, in_w=100, stride_h=2), (16, 16), _lib.ERR_INVALID_ARGUMENT, "stride-1"),
+    (dict(in_h=100, in_w=100), (16, 0), _lib.ERR_INVALID_ARGUMENT, "both tile sizes"),
+])
+def test_tiled_plan_rejections(kw, tile, code, text):
+    with pytest.raises(_lib.FbfcError) as e:
+        _q(**dict(kw, tile_h=tile[0], tile_w=tile[1]))
+    assert e.value.code == code
+    assert text in e.value.message
+
+
+def test_tiled_plan_accepts_images_too_large_for_one_fft():
+    with pytest.raises(_lib.FbfcError):
+        _q(in_h=224, in_w=224)
+    assert _q(in_h=224, in_w=224, tile_h=32, tile_w=32).fft_size == 32
