@@ -218,6 +218,43 @@ def measure_reuse_step(nn, torch, synth, steps, warmup):
     return {"ms_per_step": ms, "effective_tflops": 3 * 2.0 * B * F * P * o * o * k * k / (ms * 1e-3) / 1e12}
 
 
+def measure_tiled(nn, torch, synth, steps, warmup):
+    """A VGG-like layer (batch 64, 64 -> 128 planes, 112 x 112, 3 x 3, pad 1; the reference's tiled
+    benchmark shape, test/test_FFT.lua:466-467) through the tiled modules (tiles 32 and 16) and, for
+    comparison, through one FFT of size 128 per plane."""
+    B, P, F, H, k, pad, seed = 64, 64, 128, 112, 3, 1, 1006
+    o = H + 2 * pad - k + 1
+    flop_pass = 2.0 * B * F * P * o * o * k * k
+    x = torch.from_numpy(synth.uniform(seed, (B, P, H, H), stream=0)).cuda()
+    g = torch.from_numpy(synth.uniform(seed, (B, F, o, o), stream=3)).cuda()
+    w = torch.from_numpy(synth.normal(seed, (F, P, k, k), 0.0, 0.05, stream=1)).cuda()
+    out = {"workload": "vgg_like_b64_64x128_112x112_k3_p1", "gflop_per_pass": flop_pass / 1e9, "variants": {}}
+    passes = ("fprop", "bprop", "accgrad")
+    for name, tile in (("tile32", 32), ("tile16", 16), ("untiled_fft128", None)):
+        if tile is None:
+            net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad)
+        else:
+            net = nn.SpatialConvolutionFFTTiled(P, F, k, k, 1, 1, pad, pad, tile, tile)
+        net.weight.copy_(w)
+        net.bias.zero_()
+        n = max(3, steps // 5)
+        entry = {"ms_per_step": time_loop(torch, lambda: [run_pass(net, x, g, p) for p in passes], n, 2)}
+        entry["effective_tflops"] = 3 * flop_pass / (entry["ms_per_step"] * 1e-3) / 1e12
+        entry["ms_per_pass"] = {p: time_loop(torch, lambda: run_pass(net, x, g, p), n, 1) for p in passes}
+        net.timed = 3
+        entry["stage_ms"] = {}
+        for p in passes:
+            run_pass(net, x, g, p)
+            entry["stage_ms"][p] = {s: v for s, v in net.stageTimes(x).items() if v > 0}
+        net.timed = False
+        plan = net._plan_for(B, H, H)
+        entry["fft_size"] = plan.info.fft_size
+        entry["tiles"] = [plan.info.tiles_h, plan.info.tiles_w]
+        net.cleanupBuffers()
+        out["variants"][name] = entry
+    return out
+
+
 def measure_copy_bandwidth(torch):
     """A plain 256 MiB device-to-device copy: what HBM delivers to a trivial kernel on this box."""
     a = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
@@ -322,6 +359,7 @@ def main():
             if name != MAIN:
                 others[name] = measure_config(nn, torch, synth, name, max(5, args.steps // 5), 2)
         others["config2_fft_round_trip_8192x32x32"] = measure_fft_round_trip(nn, torch, synth, args.steps, args.warmup)
+        others["tiled_convolution"] = measure_tiled(nn, torch, synth, args.steps, args.warmup)
         line["other_configs"] = others
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)
     print(json.dumps(line))

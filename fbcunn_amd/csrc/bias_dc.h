@@ -21,8 +21,17 @@ __device__ __forceinline__ void bias_grad_dc_body(const BiasGradJob &j, unsigned
     const int fl = threadIdx.x & 63, slice = threadIdx.x >> 6;
     const int f = (int)block * 64 + fl;
     float acc = 0.0f;
-    if (f < j.planes)
-        for (int b = slice; b < j.batch; b += 4) acc += j.dc[(long)b * j.planes + f].x;
+    if (f < j.planes) {
+        // eight loads in flight per lane: a tiled plan sums over batch * tiles planes
+        float a[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        int b = slice;
+        for (; b + 28 < j.batch; b += 32) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) a[u] += j.dc[(long)(b + 4 * u) * j.planes + f].x;
+        }
+        for (; b < j.batch; b += 4) a[0] += j.dc[(long)b * j.planes + f].x;
+        acc = ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+    }
     part[slice][fl] = acc;
     __syncthreads();
     if (slice == 0 && f < j.planes)

@@ -159,27 +159,51 @@ __device__ __forceinline__ void build_window_table(int4 *tbl, const Window &win,
     }
 }
 
-// nrows = nph * h canvas rows of the planes [first, first + nph) of the workgroup
+// Moves the windows of planes [first, first + nph) of the workgroup between global memory and their
+// nph * h canvas rows.  Each wave takes every fourth plane, so the window corner and the plane's base
+// address are wave-uniform; its lanes sweep the window 64 elements (N <= 32: at least two rows) at a
+// time with all loads of a plane in flight together.
 template <int N, bool TO_LDS>
 __device__ __forceinline__ void copy_windows(float *smem, float *g, const int4 *tbl, int first, int nph,
                                              int h, int w, int padL, const Window &win, int tid)
 {
     constexpr int LDR = Canvas<N>::LDR;
-    const int total = nph * h * N;
-    const int magic = (1 << 20) / h + 1;  // rr / h for rr < 512 <= T * h
-    for (int e = tid; e < total; e += 256) {
-        const int c = e % N, rr = e / N;
-        const int tl = (rr * magic) >> 20;
-        const int r = rr - tl * h;
+    constexpr int ITER = (N * N) / 64;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int c = lane % N, r0 = lane / N;
+    for (int tl = wave; tl < nph; tl += 4) {
         const int4 q = tbl[first + tl];
-        const int y = q.z + r, x = q.w + c;
-        const bool ok = (c < w) && ((unsigned)y < (unsigned)win.img_h) && ((unsigned)x < (unsigned)win.img_w);
-        float *gp = g + ((((long)q.y) << 32) | (long)(unsigned)q.x) + (long)y * win.img_w + x;
-        float *sp = smem + rr * LDR + padL + c;
+        const int off_lo = __builtin_amdgcn_readfirstlane(q.x), off_hi = __builtin_amdgcn_readfirstlane(q.y);
+        const int y0 = __builtin_amdgcn_readfirstlane(q.z), x0 = __builtin_amdgcn_readfirstlane(q.w);
+        float *gp = g + ((((long)off_hi) << 32) | (long)(unsigned)off_lo) + x0 + c;
+        float *sp = smem + (tl * h) * LDR + padL + c;
+        const bool xok = (c < w) && ((unsigned)(x0 + c) < (unsigned)win.img_w);
+        float v[ITER];
         if (TO_LDS) {
-            *sp = ok ? *gp : 0.0f;
-        } else if (ok) {
-            *gp = *sp;
+#pragma unroll
+            for (int i = 0; i < ITER; ++i) {
+                const int r = r0 + i * (64 / N);
+                const int y = y0 + r;
+                const bool ok = xok && (r < h) && ((unsigned)y < (unsigned)win.img_h);
+                v[i] = ok ? gp[(long)y * win.img_w] : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < ITER; ++i) {
+                const int r = r0 + i * (64 / N);
+                if (r < h) sp[r * LDR] = v[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < ITER; ++i) {
+                const int r = r0 + i * (64 / N);
+                v[i] = (r < h) ? sp[r * LDR] : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < ITER; ++i) {
+                const int r = r0 + i * (64 / N);
+                const int y = y0 + r;
+                if (xok && (r < h) && ((unsigned)y < (unsigned)win.img_h)) gp[(long)y * win.img_w] = v[i];
+            }
         }
     }
 }
