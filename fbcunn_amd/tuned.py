@@ -1,0 +1,174 @@
+"""Host-side mirror of fbnn.SpatialConvolution (fbcunn/SpatialConvolution.lua): the front
+that, on the first updateOutput, times the FFT strategies that fit the layer and keeps the
+fastest (:188-422).  The reference also times cuDNN and falls back to it; this build has
+no direct-convolution path, so the candidates are the FFT strategies only and a layer none
+of them can run (stride above 1, sizes out of range) raises.
+"""
+import time
+
+import torch
+
+from . import _lib
+from . import modules as nn
+
+__all__ = ["SpatialConvolution"]
+
+
+def _time_function(fn, *args):
+    """3 trials, the first dropped, mean of the rest in ms (SpatialConvolution.lua:98-112)."""
+    num_trials, total = 3, 0.0
+    torch.cuda.synchronize()
+    for i in range(num_trials):
+        t0 = time.perf_counter()
+        fn(*args)
+        torch.cuda.synchronize()
+        if i > 0:
+            total += time.perf_counter() - t0
+    return total / (num_trials - 1) * 1e3
+
+
+class SpatialConvolution:
+    """fbnn.SpatialConvolution(nInputPlane, nOutputPlane, kW, kH, dW, dH, padLeft, padUp,
+    maximalMemoryOverhead, inferenceOnly)."""
+
+    reportErrors = False
+
+    def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padLeft=0, padUp=0,
+                 maximalMemoryOverhead=None, inferenceOnly=False, device="cuda"):
+        self.inputPlanes, self.outputPlanes = nInputPlane, nOutputPlane
+        self.kW, self.kH, self.dW, self.dH = kW, kH, dW, dH
+        self.padLeft, self.padUp = padLeft, padUp
+        self.maximalMemoryOverhead = maximalMemoryOverhead
+        self.inferenceOnly = bool(inferenceOnly)
+        self.reportLevel = 0
+        self.device = torch.device(device)
+        # parameters live here and are handed to the strategy that wins
+        holder = nn.SpatialConvolutionFBFFT(nInputPlane, nOutputPlane, kW, kH, 1, 1, 0, 0, device=device) \
+            if (dW == 1 and dH == 1) else None
+        if holder is None:
+            raise ValueError("fft only supports stride-1 convolutions atm (and there is no direct path here)")
+        self.weight, self.bias = holder.weight, holder.bias
+        self.gradWeight, self.gradBias = holder.gradWeight, holder.gradBias
+        self.output = None
+        self.gradInput = None
+        self.bestModuleInst = None
+        self.timings = {}
+
+    def setInferenceOnly(self, val):
+        assert isinstance(val, bool)
+        self.inferenceOnly = val
+
+    # -- candidates (SpatialConvolution.lua:237-300) -----------------------------------
+    def _candidates(self, iH, iW):
+        reuse_all, reuse_none = nn.SpatialConvolutionFFT.memoryReuseAll, nn.SpatialConvolutionFFT.memoryReuseNone
+        cands = [("SpatialConvolutionFBFFT", None, reuse_all), ("SpatialConvolutionFBFFT", None, reuse_none)]
+        if self.kH <= 9 and self.kW <= 9:
+            tiles = (16, 32)
+        else:
+            tiles = (32,)
+        for t in tiles:
+            for reuse in (reuse_none, reuse_all):
+                cands.append(("SpatialConvolutionFFTTiled", t, reuse))
+        return cands
+
+    def _plan_bytes(self, batch, iH, iW, tile, reuse):
+        """Frequency-buffer bytes the strategy would allocate, or None if it cannot run."""
+        kw = dict(batch=batch, in_planes=self.inputPlanes, out_planes=self.outputPlanes, in_h=iH, in_w=iW,
+                  k_h=self.kH, k_w=self.kW, stride_h=self.dH, stride_w=self.dW, pad_h=self.padUp,
+                  pad_w=self.padLeft)
+        try:
+            info = _lib.plan_query(tile_h=tile or 0, tile_w=tile or 0, **kw)
+        except _lib.FbfcError:
+            return None
+        sizes = (info.input_freq_bytes, info.weight_freq_bytes, info.output_freq_bytes)
+        return sum(sizes) + (max(sizes) if reuse != nn.SpatialConvolutionFFT.memoryReuseNone else 0)
+
+    def _make(self, cls, tile, reuse):
+        args = (self.inputPlanes, self.outputPlanes, self.kW, self.kH, self.dW, self.dH, self.padLeft, self.padUp)
+        if tile is None:
+            inst = getattr(nn, cls)(*args, reuse, device=self.device)
+        else:
+            inst = getattr(nn, cls)(*args, tile, tile, reuse, device=self.device)
+        inst.weight, inst.bias = self.weight, self.bias
+        inst.gradWeight, inst.gradBias = self.gradWeight, self.gradBias
+        return inst
+
+    def _tune(self, input):
+        B, _, iH, iW = input.shape
+        oH = iH + 2 * self.padUp - self.kH + 1
+        oW = iW + 2 * self.padLeft - self.kW + 1
+        grad_output = torch.zeros(B, self.outputPlanes, max(oH, 1), max(oW, 1), device=input.device)
+        # tuning must not disturb the caller's gradients
+        keep_gw, keep_gb = self.gradWeight.clone(), self.gradBias.clone()
+        best, best_ms = None, float("inf")
+        self.timings = {}
+        for cls, tile, reuse in self._candidates(iH, iW):
+            nbytes = self._plan_bytes(B, iH, iW, tile, reuse)
+            key = (cls, tile, reuse)
+            if nbytes is None:
+                self.timings[key] = None          # the strategy cannot run this layer
+                continue
+            if self.maximalMemoryOverhead is not None and nbytes > self.maximalMemoryOverhead:
+                self.timings[key] = {"memoryConsumption": nbytes, "skipped": "exceeds maximalMemoryOverhead"}
+                continue
+            inst = self._make(cls, tile, reuse)
+            try:
+                t1 = _time_function(inst.updateOutput, input)
+                t2 = t3 = 0.0
+                if not self.inferenceOnly:
+                    t2 = _time_function(inst.updateGradInput, input, grad_output)
+                    t3 = _time_function(inst.accGradParameters, input, grad_output, 1.0)
+            except _lib.FbfcError as err:
+                if self.reportErrors:
+                    print("%s tile %s: %s" % (cls, tile, err))
+                inst.cleanupBuffers()
+                self.timings[key] = None
+                continue
+            self.timings[key] = {"memoryConsumption": nbytes, "ms": (t1, t2, t3)}
+            if t1 + t2 + t3 < best_ms:
+                if best is not None:
+                    best.cleanupBuffers()
+                best, best_ms = inst, t1 + t2 + t3
+                self.bestKey = key
+            else:
+                inst.cleanupBuffers()
+        self.gradWeight.copy_(keep_gw)
+        self.gradBias.copy_(keep_gb)
+        if best is None:
+            raise _lib.FbfcError(_lib.ERR_UNSUPPORTED_SIZE,
+                                 "no FFT strategy can run this layer (and there is no direct path here)")
+        if self.reportLevel >= 1:
+            print("Best FFT: ", best_ms, " ", self.bestKey)
+        self.bestModuleInst = best
+        self.batchSize, self.iH, self.iW = B, iH, iW
+
+    # -- nn.Module protocol --------------------------------------------------------------
+    def updateOutput(self, input):
+        if input.dim() != 4:
+            raise ValueError("Only supports 4-D tensors atm")
+        if self.bestModuleInst is None:
+            self._tune(input)
+        if (self.batchSize, self.iH, self.iW) != (input.size(0), input.size(2), input.size(3)):
+            raise ValueError("tuned for %s, got %s" % ((self.batchSize, self.iH, self.iW), tuple(input.shape)))
+        self.bestModuleInst.weight, self.bestModuleInst.bias = self.weight, self.bias
+        self.output = self.bestModuleInst.updateOutput(input)
+        return self.output
+
+    forward = updateOutput
+
+    def updateGradInput(self, input, gradOutput):
+        assert self.bestModuleInst is not None, "Must have been tuned in updateOutput already!"
+        assert not self.inferenceOnly, "Inference only specified => no gradInput "
+        self.gradInput = self.bestModuleInst.updateGradInput(input, gradOutput)
+        return self.gradInput
+
+    def accGradParameters(self, input, gradOutput, scale=1.0):
+        assert self.bestModuleInst is not None, "Must have been tuned in updateOutput already!"
+        assert not self.inferenceOnly, "Inference only specified => no accGrads "
+        self.bestModuleInst.gradWeight, self.bestModuleInst.gradBias = self.gradWeight, self.gradBias
+        self.bestModuleInst.accGradParameters(input, gradOutput, scale)
+
+    def cleanupBuffers(self):
+        if self.bestModuleInst is not None:
+            self.bestModuleInst.cleanupBuffers()
+        self.bestModuleInst = None

@@ -37,6 +37,13 @@ def lib():
     return _lib
 
 
+def set_threads(n):
+    """OpenMP threads of the parallel loops from now on (n < 1: unchanged); returns the count in effect."""
+    fn = lib().orc_set_threads
+    fn.argtypes, fn.restype = [ctypes.c_int], ctypes.c_int
+    return int(fn(int(n)))
+
+
 def _p(a):
     return a.ctypes.data_as(_f32p)
 

@@ -38,12 +38,28 @@
  * brute-force loops on tiny shapes.
  */
 #include <math.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 #include <stddef.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
 
 #define IDX4(a, b, c, d, B, C, D) ((((size_t)(a) * (B) + (b)) * (C) + (c)) * (D) + (d))
+
+/* Threads the parallel loops use from now on (n < 1: leave as is); returns the count in effect.
+ * Only the timing of the CPU baseline uses it. */
+int orc_set_threads(int n)
+{
+#ifdef _OPENMP
+    if (n >= 1) omp_set_num_threads(n);
+    return omp_get_max_threads();
+#else
+    (void)n;
+    return 1;
+#endif
+}
 
 long orc_valid_conv_size(long in, long k, long stride) { return (in - k) / stride + 1; }
 long orc_valid_rev_conv_size(long in, long k, long stride) { return in - (k - 1) * stride; }
