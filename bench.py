@@ -62,6 +62,9 @@ def stage_model(cfg, pass_, n, q):
 # (profiles/hbm_traffic_all_configs.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, the
 # factors a 256 MiB device copy gives for the same counters (--calibrate-copy).
 MEASURED_TRAFFIC_MAIN = {
+    "cgemm_hybrid_kernel<0>": (18462 * 2.0 + 18432) * 1024,   # same operands and result as the
+    "cgemm_hybrid_kernel<1>": (18462 * 2.0 + 18432) * 1024,   # split-K kernel it replaced; to be
+    "cgemm_hybrid_kernel<2>": (18463 * 2.0 + 18432) * 1024,   # re-measured with the next counter run
     "cgemm_splitk_kernel<0, 4>": (18462 * 2.0 + 18432) * 1024,
     "cgemm_splitk_kernel<1, 4>": (18462 * 2.0 + 18432) * 1024,
     "cgemm_splitk_kernel<2, 4>": (18463 * 2.0 + 18432) * 1024,
@@ -78,6 +81,11 @@ def mm_kernel_name(pass_, q, m, n, k):
     mode = {"fprop": 0, "bprop": 1, "accgrad": 2}[pass_]
     tiles64 = q * ((m + 63) // 64) * ((n + 63) // 64)
     direct_ok = m % 64 == 0 and n % 64 == 0 and k % 16 == 0
+    if direct_ok and k % 64 == 0 and 256 <= tiles64 < 4 * 256:
+        t64 = (m // 64) * (n // 64)
+        q_direct = (tiles64 // 256) * 256 // t64
+        if 0 < q_direct < q:
+            return "cgemm_hybrid_kernel<%d>" % mode
     if direct_ok and tiles64 >= 4 * 256:
         return "cgemm_ldsdirect_kernel<%d>" % mode
     if m % 32 == 0 and n % 32 == 0 and k % 16 == 0:

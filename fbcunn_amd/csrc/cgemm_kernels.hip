@@ -238,22 +238,20 @@ __device__ __forceinline__ void lds_direct_tile(const float2 *__restrict__ Mq, i
     }
 }
 
+// One 64x64 tile, workgroup index wg = frequency * tiles + tile.  lds: 4 operand tiles of 8 KB
+// (A and B, double-buffered).
 template <int MODE>
-__global__ __launch_bounds__(256) void cgemm_ldsdirect_kernel(const float2 *__restrict__ A,
-                                                              const float2 *__restrict__ B,
-                                                              float2 *__restrict__ C, int M, int N,
-                                                              int K, float alpha, int accumulate,
-                                                              int tilesM, int tilesN, int total_wgs,
-                                                              int chunk)
+__device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restrict__ A,
+                                               const float2 *__restrict__ B, float2 *__restrict__ C,
+                                               int M, int N, int K, float alpha, int accumulate,
+                                               int tilesM, int tilesN, int wg)
 {
     constexpr bool A_KC = (MODE != 2);
     constexpr bool B_KC = (MODE == 0);
     constexpr int TILE = 64 * KT * 2;  // floats per operand tile (8 KB)
-    __shared__ __align__(16) float As[2][TILE];
-    __shared__ __align__(16) float Bs[2][TILE];
+    float *const As[2] = {lds, lds + TILE};
+    float *const Bs[2] = {lds + 2 * TILE, lds + 3 * TILE};
 
-    const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
-    if (wg >= total_wgs) return;
     const int tiles = tilesM * tilesN;
     const int q = wg / tiles;
     const int tile = wg - q * tiles;
@@ -360,6 +358,22 @@ __global__ __launch_bounds__(256) void cgemm_ldsdirect_kernel(const float2 *__re
     }
 }
 
+constexpr int LDSDIRECT_FLOATS = 4 * 64 * KT * 2;  // 32 KB
+
+template <int MODE>
+__global__ __launch_bounds__(256) void cgemm_ldsdirect_kernel(const float2 *__restrict__ A,
+                                                              const float2 *__restrict__ B,
+                                                              float2 *__restrict__ C, int M, int N,
+                                                              int K, float alpha, int accumulate,
+                                                              int tilesM, int tilesN, int total_wgs,
+                                                              int chunk)
+{
+    __shared__ __align__(16) float lds[LDSDIRECT_FLOATS];
+    const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
+    if (wg >= total_wgs) return;
+    ldsdirect_body<MODE>(lds, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, wg);
+}
+
 // ---------------------------------------------------------------------------------------
 // Split-K kernel for small problems (few 64x64 tiles per CU).
 //
@@ -437,19 +451,14 @@ __device__ __forceinline__ void splitk_mfma(const float (&a)[16], const float (&
     }
 }
 
+// red: [wave][accumulator register][lane] partial sums (used when SK > 1)
 template <int MODE, int SK>
-__global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restrict__ A,
-                                                           const float2 *__restrict__ B,
-                                                           float2 *__restrict__ C, int M, int N, int K,
-                                                           float alpha, int accumulate, int tilesM,
-                                                           int tilesN, int total_tiles, int total_wgs,
-                                                           int chunk)
+__device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *__restrict__ A,
+                                            const float2 *__restrict__ B, float2 *__restrict__ C, int M,
+                                            int N, int K, float alpha, int accumulate, int tilesM,
+                                            int tilesN, int total_tiles, int wg)
 {
     constexpr int TPW = 4 / SK;  // 32x32 blocks per workgroup; SK waves share one block's K range
-    __shared__ float red[SK > 1 ? 4 : 1][32][64];  // [wave][accumulator register][lane]
-
-    const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
-    if (wg >= total_wgs) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 31, h = lane >> 5;
     const int ks = wave % SK;  // which share of K
@@ -551,6 +560,51 @@ __global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restr
 }
 
 template <int MODE, int SK>
+__global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restrict__ A,
+                                                           const float2 *__restrict__ B,
+                                                           float2 *__restrict__ C, int M, int N, int K,
+                                                           float alpha, int accumulate, int tilesM,
+                                                           int tilesN, int total_tiles, int total_wgs,
+                                                           int chunk)
+{
+    __shared__ float red[SK > 1 ? 4 : 1][32][64];
+    const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
+    if (wg >= total_wgs) return;
+    splitk_body<MODE, SK>(red, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, total_tiles, wg);
+}
+
+// ---------------------------------------------------------------------------------------
+// Hybrid launch for problems of a few 64x64 tiles per CU.  Whole rounds of tiles (a multiple of
+// the 256 CUs) run as LDS-direct tiles; the frequencies left over, which would make a last round
+// that fills only part of the chip, run as 32x32 blocks whose K range is split over the four
+// waves of a workgroup, so that every CU gets the same share of them.  Workgroups of the first
+// kind come first in dispatch order.  Both bodies use the same 32 KB of LDS.
+// ---------------------------------------------------------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(256) void cgemm_hybrid_kernel(const float2 *__restrict__ A,
+                                                           const float2 *__restrict__ B,
+                                                           float2 *__restrict__ C, int M, int N, int K,
+                                                           float alpha, int accumulate, int q_direct,
+                                                           int direct_wgs, int chunk_direct,
+                                                           int split_tiles, int split_wgs, int chunk_split)
+{
+    __shared__ __align__(16) float lds[LDSDIRECT_FLOATS];
+    static_assert(LDSDIRECT_FLOATS == 4 * 32 * 64, "both bodies share one buffer");
+    const int x = (int)(blockIdx.x % 8), j = (int)(blockIdx.x / 8);
+    if (j < chunk_direct) {
+        const int wg = x * chunk_direct + j;
+        if (wg >= direct_wgs) return;
+        ldsdirect_body<MODE>(lds, A, B, C, M, N, K, alpha, accumulate, M / 64, N / 64, wg);
+    } else {
+        const int wg = x * chunk_split + (j - chunk_direct);
+        if (wg >= split_wgs) return;
+        const long off = (long)q_direct;  // the split part starts at frequency q_direct
+        splitk_body<MODE, 4>(reinterpret_cast<float (*)[32][64]>(lds), A + off * M * K, B + off * N * K,
+                             C + off * M * N, M, N, K, alpha, accumulate, M / 32, N / 32, split_tiles, wg);
+    }
+}
+
+template <int MODE, int SK>
 static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_freq, int m, int n,
                                 int k, float alpha, int accumulate, hipStream_t s)
 {
@@ -566,7 +620,8 @@ static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_
 }
 
 // FBFC_CGEMM_SPLITK forces a kernel variant (for measurements): 0 = register-staged LDS tiles,
-// 8 = LDS-direct tiles, 1 / 2 / 4 = register-fed kernel with that many waves per block.
+// 8 = LDS-direct tiles, 9 = hybrid of LDS-direct tiles and split blocks, 1 / 2 / 4 = register-fed
+// kernel with that many waves per block.
 static int splitk_override()
 {
     static int v = -2;
@@ -593,6 +648,24 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
     const int force = splitk_override();
     const bool direct_ok = (m % 64) == 0 && (n % 64) == 0 && (k % 16) == 0 && aligned16;
     const long tot32 = (long)n_freq * (m / 32) * (n / 32);
+    // fewer than four rounds of tiles and a ragged last one: whole rounds as tiles, the rest as split
+    // blocks (measured: 28 vs 31 us at 144 x 128^3; with four or more rounds plain tiles are as fast)
+    if (direct_ok && (k % 64) == 0 && (force == 9 || (force < 0 && total >= 256 && total < 4 * 256))) {
+        const int t64 = tilesM * tilesN;
+        const int q_direct = (int)((total / 256) * 256 / t64);
+        const int q_split = n_freq - q_direct;
+        if (q_split > 0 && q_direct > 0) {
+            const int direct_wgs = q_direct * t64;
+            const int split_tiles = q_split * (m / 32) * (n / 32);  // one workgroup per 32x32 block
+            const int chunk_direct = (direct_wgs + 7) / 8, chunk_split = (split_tiles + 7) / 8;
+            hipLaunchKernelGGL(cgemm_hybrid_kernel<MODE>, dim3((unsigned)((chunk_direct + chunk_split) * 8)),
+                               dim3(256), 0, s, reinterpret_cast<const float2 *>(A),
+                               reinterpret_cast<const float2 *>(B), reinterpret_cast<float2 *>(C), m, n, k,
+                               alpha, accumulate, q_direct, direct_wgs, chunk_direct, split_tiles,
+                               split_tiles, chunk_split);
+            return hipGetLastError();
+        }
+    }
     const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && total >= 4 * 256));
     if (!prefer_direct && (m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 &&
         tot32 * 4 < 0x7fffff00L) {

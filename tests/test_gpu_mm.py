@@ -29,6 +29,9 @@ SHAPES = [  # Q, m, n, k
     (2, 65, 33, 17), (3, 70, 130, 40), (2, 64, 256, 96), (9, 16, 16, 4), (2, 100, 20, 129),
     # small aligned problems take the split-K kernel (M, N multiples of 32, K of 64)
     (4, 32, 32, 64), (2, 96, 160, 128), (3, 128, 128, 128), (5, 64, 32, 192), (144, 128, 128, 128),
+    # a few rounds of 64x64 tiles with a ragged last one: whole rounds as LDS-direct tiles, the
+    # left-over frequencies as split blocks, in one launch
+    (70, 128, 128, 64), (300, 64, 64, 128), (33, 192, 128, 64),
 ]
 
 
@@ -52,7 +55,7 @@ def test_transpose_mm(nn, mode, Q, m, n, k):
     assert np.abs(got - want).max() <= TOL * np.abs(want).max()
 
 
-@pytest.mark.parametrize("Q,m,n,k", [(3, 40, 50, 20), (3, 64, 96, 64)])
+@pytest.mark.parametrize("Q,m,n,k", [(3, 40, 50, 20), (3, 64, 96, 64), (70, 128, 128, 64)])
 def test_accumulate_flag(nn, Q, m, n, k):
     A, B = synth.uniform(3, (Q, m, k, 2)), synth.uniform(4, (Q, k, n, 2))
     C0 = synth.uniform(5, (Q, m, n, 2))
