@@ -81,7 +81,7 @@ def mm_kernel_name(pass_, q, m, n, k):
     mode = {"fprop": 0, "bprop": 1, "accgrad": 2}[pass_]
     tiles64 = q * ((m + 63) // 64) * ((n + 63) // 64)
     direct_ok = m % 64 == 0 and n % 64 == 0 and k % 16 == 0
-    if direct_ok and k % 64 == 0 and 256 <= tiles64 < 4 * 256:
+    if direct_ok and k % 64 == 0 and 256 <= tiles64 < 8 * 256 and tiles64 % 256 <= 128:
         t64 = (m // 64) * (n // 64)
         q_direct = (tiles64 // 256) * 256 // t64
         if 0 < q_direct < q:

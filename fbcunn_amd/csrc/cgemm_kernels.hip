@@ -249,8 +249,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
     constexpr bool A_KC = (MODE != 2);
     constexpr bool B_KC = (MODE == 0);
     constexpr int TILE = 64 * KT * 2;  // floats per operand tile (8 KB)
-    float *const As[2] = {lds, lds + TILE};
-    float *const Bs[2] = {lds + 2 * TILE, lds + 3 * TILE};
+    // buffer b of A at lds + b * TILE, of B at lds + (2 + b) * TILE
 
     const int tiles = tilesM * tilesN;
     const int q = wg / tiles;
@@ -273,10 +272,11 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
     const int nk = K / KT;
     auto issue = [&](int kt, int buf) {
         const int k0 = kt * KT;
-        if (A_KC) lds_direct_tile<true>(Aq, K, m0, k0, As[buf], wave, lane);   // A[m][k]
-        else      lds_direct_tile<false>(Aq, M, k0, m0, As[buf], wave, lane);  // A[k][m]
-        if (B_KC) lds_direct_tile<true>(Bq, K, n0, k0, Bs[buf], wave, lane);   // B[n][k]
-        else      lds_direct_tile<false>(Bq, N, k0, n0, Bs[buf], wave, lane);  // B[k][n]
+        float *ab = lds + buf * TILE, *bb = lds + (2 + buf) * TILE;
+        if (A_KC) lds_direct_tile<true>(Aq, K, m0, k0, ab, wave, lane);   // A[m][k]
+        else      lds_direct_tile<false>(Aq, M, k0, m0, ab, wave, lane);  // A[k][m]
+        if (B_KC) lds_direct_tile<true>(Bq, K, n0, k0, bb, wave, lane);   // B[n][k]
+        else      lds_direct_tile<false>(Bq, N, k0, n0, bb, wave, lane);  // B[k][n]
     };
 
     issue(0, 0);
@@ -292,8 +292,8 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
         const int buf = kt & 1;
         if (kt + 1 < nk) issue(kt + 1, buf ^ 1);  // asynchronous: lands while this tile is multiplied
 
-        const float *as = As[buf];
-        const float *bs = Bs[buf];
+        const float *as = lds + buf * TILE;
+        const float *bs = lds + (2 + buf) * TILE;
         if (MODE == 0) {
             float a[16], b[16];
 #pragma unroll
@@ -648,9 +648,11 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
     const int force = splitk_override();
     const bool direct_ok = (m % 64) == 0 && (n % 64) == 0 && (k % 16) == 0 && aligned16;
     const long tot32 = (long)n_freq * (m / 32) * (n / 32);
-    // fewer than four rounds of tiles and a ragged last one: whole rounds as tiles, the rest as split
-    // blocks (measured: 28 vs 31 us at 144 x 128^3; with four or more rounds plain tiles are as fast)
-    if (direct_ok && (k % 64) == 0 && (force == 9 || (force < 0 && total >= 256 && total < 4 * 256))) {
+    // A few rounds of tiles whose last round would fill at most half the chip: whole rounds as tiles,
+    // the rest as split blocks (measured: 25 vs 31 us at 144 x 128^3, 28.4 vs 30.5 at 544 x 128x64x64;
+    // with a fuller last round plain tiles are as fast).
+    if (direct_ok && (k % 64) == 0 &&
+        (force == 9 || (force < 0 && total >= 256 && total < 8 * 256 && total % 256 <= 128))) {
         const int t64 = tilesM * tilesN;
         const int q_direct = (int)((total / 256) * 256 / t64);
         const int q_split = n_freq - q_direct;

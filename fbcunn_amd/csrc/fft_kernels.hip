@@ -222,7 +222,9 @@ struct FwdJob {
     Window win;
 };
 
-template <int N, bool WIN>
+// NZ < N: planes of at most NZ x NZ at the canvas origin (convolution kernels): the transforms skip
+// the inputs that are known to be zero.
+template <int N, bool WIN, int NZ>
 __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(FwdJob job0, FwdJob job1,
                                                                       unsigned blocks0)
 {
@@ -285,9 +287,14 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
             const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? tl * h + ib : zrow) * LDR);
             static_for<N / 4>([&](auto jj) {
                 constexpr int j = decltype(jj)::value;
-                const float4 a = pa[j], b = pb[j];
-                re[4 * j] = a.x; re[4 * j + 1] = a.y; re[4 * j + 2] = a.z; re[4 * j + 3] = a.w;
-                im[4 * j] = b.x; im[4 * j + 1] = b.y; im[4 * j + 2] = b.z; im[4 * j + 3] = b.w;
+                if constexpr (4 * j < NZ) {
+                    const float4 a = pa[j], b = pb[j];
+                    re[4 * j] = a.x; re[4 * j + 1] = a.y; re[4 * j + 2] = a.z; re[4 * j + 3] = a.w;
+                    im[4 * j] = b.x; im[4 * j + 1] = b.y; im[4 * j + 2] = b.z; im[4 * j + 3] = b.w;
+                } else {
+                    re[4 * j] = re[4 * j + 1] = re[4 * j + 2] = re[4 * j + 3] = 0.0f;
+                    im[4 * j] = im[4 * j + 1] = im[4 * j + 2] = im[4 * j + 3] = 0.0f;
+                }
             });
         }
     });
@@ -303,7 +310,7 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
     __syncthreads();  // staging area fully consumed; the tile may overwrite it
     if (tid < S::KXP * T) R[nrows * S::ROWSTRIDE + tid] = make_float2(0.0f, 0.0f);
     if (row_active) {
-        fft_inplace<N, false>(re, im);
+        fft_inplace_nz<N, NZ, false>(re, im);
         float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
         float2 *Rb = Ra + S::ROWSTRIDE;
         Ra[0] = make_float2(re[brev<N>(0)], re[brev<N>(N / 2)]);
@@ -346,18 +353,23 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
             const float2 *col = R + kl * T + t;
             static_for<N>([&](auto yy) {
                 constexpr int y = decltype(yy)::value;
-                // canvas rows outside the plane read the zero row (uniform select, no branch)
-                const int row = ((y >= y_lo) && (y < y_hi)) ? (y - y_lo) : nrows;
-                const float2 v = col[row * S::ROWSTRIDE];
-                re[y] = v.x;
-                im[y] = v.y;
+                if constexpr (y < NZ) {
+                    // canvas rows outside the plane read the zero row (uniform select, no branch)
+                    const int row = ((y >= y_lo) && (y < y_hi)) ? (y - y_lo) : nrows;
+                    const float2 v = col[row * S::ROWSTRIDE];
+                    re[y] = v.x;
+                    im[y] = v.y;
+                } else {
+                    re[y] = 0.0f;
+                    im[y] = 0.0f;
+                }
             });
         }
     });
 
     // ---- column FFT and frequency-major store, all lanes at once ----
     if (t < np) {
-        fft_inplace<N, false>(re, im);
+        fft_inplace_nz<N, NZ, false>(re, im);
         // address = uniform base (frequency row ky, first plane of the group) + 32-bit lane offset
         const unsigned voff = (unsigned)(((long)kx * planes + t) * (long)sizeof(float2));
         const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + t) * (long)sizeof(float2));
@@ -583,12 +595,12 @@ static bool window_ok(const Window &w, long planes, int h, int ww)
 }
 
 // second == nullptr: one tensor only
-template <int N, bool WIN>
+template <int N, bool WIN, int NZ = N>
 static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
 {
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rfft2d_kernel<N, WIN>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rfft2d_kernel<N, WIN, NZ>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         attr_done = true;
@@ -609,7 +621,7 @@ static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_
         lds += FftShape<N>::T * sizeof(int4);
     }
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((rfft2d_kernel<N, WIN>), dim3((unsigned)blocks), dim3(256), lds, s, j0, j1,
+    hipLaunchKernelGGL((rfft2d_kernel<N, WIN, NZ>), dim3((unsigned)blocks), dim3(256), lds, s, j0, j1,
                        (unsigned)blocks0);
     return hipGetLastError();
 }
@@ -656,6 +668,16 @@ static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStr
             case 32: return launch_fwd<32, true>(a, b, s);
             default: return hipErrorInvalidValue;
         }
+    }
+    if (N == 64) {
+        // planes of at most 16 x 16 at the origin (convolution kernels) take the variant that skips
+        // the zero inputs; a pair that holds such an operand is issued as two launches
+        auto small = [](const FwdArgs &x) { return x.h <= 16 && x.w <= 16 && x.padU == 0 && x.padL == 0; };
+        if (b != nullptr && (small(a) || small(*b))) {
+            const hipError_t e = dispatch_fwd(N, a, nullptr, s);
+            return e != hipSuccess ? e : dispatch_fwd(N, *b, nullptr, s);
+        }
+        if (b == nullptr && small(a)) return launch_fwd<64, false, 16>(a, nullptr, s);
     }
     switch (N) {
         case 8: return launch_fwd<8, false>(a, b, s);

@@ -106,6 +106,43 @@ __host__ __device__ __forceinline__ void fft_dif(float *re, float *im) {
     }
 }
 
+// Input-pruned variant: only the first NZ inputs of the length-LEN sequence at OFF are non-zero (the
+// caller leaves literal zeros in the others).  While half the length is at least NZ a butterfly has
+// b = 0, so a' = a and b' = a * W for the NZ leading positions and nothing at all for the others;
+// both halves then again have NZ leading non-zeros.
+template <int LEN, int OFF, int K, bool INV>
+__host__ __device__ __forceinline__ void butterfly_b0(float *re, float *im) {
+    constexpr int H = LEN / 2;
+    const float ar = re[OFF + K], ai = im[OFF + K];
+    if constexpr (K == 0) {
+        re[OFF + H] = ar;
+        im[OFF + H] = ai;
+    } else {
+        constexpr float wr = (float)cos2pi(K, LEN);
+        constexpr float wi = (float)(INV ? sin2pi(K, LEN) : -sin2pi(K, LEN));
+        re[OFF + K + H] = ar * wr - ai * wi;
+        im[OFF + K + H] = ar * wi + ai * wr;
+    }
+}
+
+template <int LEN, int OFF, bool INV, int NZ>
+__host__ __device__ __forceinline__ void fft_dif_nz(float *re, float *im) {
+    if constexpr (LEN / 2 >= NZ && LEN >= 2) {
+        static_for<NZ>([&](auto k) { butterfly_b0<LEN, OFF, decltype(k)::value, INV>(re, im); });
+        fft_dif_nz<LEN / 2, OFF, INV, NZ>(re, im);
+        fft_dif_nz<LEN / 2, OFF + LEN / 2, INV, NZ>(re, im);
+    } else {
+        fft_dif<LEN, OFF, INV>(re, im);
+    }
+}
+
+// Unnormalised length-N transform of a sequence whose inputs from NZ on are literal zeros.
+template <int N, int NZ, bool INV>
+__host__ __device__ __forceinline__ void fft_inplace_nz(float (&re)[N], float (&im)[N]) {
+    static_assert(NZ >= 1 && NZ <= N, "NZ leading non-zero inputs");
+    fft_dif_nz<N, 0, INV, NZ>(re, im);
+}
+
 // Unnormalised length-N transform in place; output index k lives at brev<N>(k).
 template <int N, bool INV>
 __host__ __device__ __forceinline__ void fft_inplace(float (&re)[N], float (&im)[N]) {

@@ -31,6 +31,7 @@ CASES = [
     (16, 7, 13, 13, 1, 1), (16, 96, 16, 16, 0, 0), (16, 33, 3, 3, 0, 0), (16, 40, 10, 12, 3, 2),
     (32, 3, 27, 27, 2, 2), (32, 48, 32, 32, 0, 0), (32, 17, 5, 5, 0, 0), (32, 35, 20, 28, 5, 1),
     (64, 9, 55, 55, 4, 4), (64, 16, 64, 64, 0, 0), (64, 5, 9, 9, 0, 0), (64, 11, 33, 40, 7, 10),
+    (64, 19, 16, 16, 0, 0), (64, 3, 1, 16, 0, 0), (64, 8, 11, 2, 0, 0), (64, 4, 9, 9, 1, 0),   # small planes: zero inputs skipped
     (128, 5, 100, 100, 3, 7), (128, 9, 128, 128, 0, 0), (128, 6, 11, 11, 0, 0), (128, 3, 70, 127, 20, 1),
 ]
 
