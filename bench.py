@@ -86,8 +86,10 @@ def mm_kernel_name(pass_, q, m, n, k):
         q_direct = (tiles64 // 256) * 256 // t64
         if 0 < q_direct < q:
             return "cgemm_hybrid_kernel<%d>" % mode
+    if mode != 1 and m % 64 == 0 and n % 96 == 0 and n % 64 != 0 and k % 16 == 0 and q * (m // 64) * (n // 96) >= 4 * 256:
+        return "cgemm_ldsdirect_kernel<%d, 3>" % mode
     if direct_ok and tiles64 >= 4 * 256:
-        return "cgemm_ldsdirect_kernel<%d>" % mode
+        return "cgemm_ldsdirect_kernel<%d, 2>" % mode
     if m % 32 == 0 and n % 32 == 0 and k % 16 == 0:
         tot32 = q * (m // 32) * (n // 32)
         if tot32 < 4096 and k % 64 == 0:
@@ -96,7 +98,7 @@ def mm_kernel_name(pass_, q, m, n, k):
             return "cgemm_splitk_kernel<%d, 2>" % mode
         return "cgemm_splitk_kernel<%d, 1>" % mode
     if direct_ok:
-        return "cgemm_ldsdirect_kernel<%d>" % mode
+        return "cgemm_ldsdirect_kernel<%d, 2>" % mode
     return "cgemm_freq_kernel<%d>" % mode
 
 

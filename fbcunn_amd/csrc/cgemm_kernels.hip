@@ -217,30 +217,36 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
 //     different bank groups (XOR swizzle instead of row padding);
 //   row-contiguous tile [16 k][32 chunks]: one instruction = 2 rows, stored as they lie.
 // ---------------------------------------------------------------------------------------
-template <bool KC>
+// ROWS = rows of a K-contiguous tile resp. columns of a row-contiguous one (64 or 96): ROWS / 8 blocks
+// of 1 KB, dealt round-robin to the NW waves of the workgroup.
+template <bool KC, int ROWS, int NW>
 __device__ __forceinline__ void lds_direct_tile(const float2 *__restrict__ Mq, int ld, int r0, int c0,
                                                 float *lds, int wave, int lane)
 {
+    constexpr int NBLK = ROWS / 8;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int blk = j * 4 + wave;  // 1 KB block of the 8 KB tile
-        const float2 *g;
-        if (KC) {  // rows r0 + 8 blk .. +7, complex k c0 .. c0+15
-            const int rl = lane >> 3, cs = lane & 7;
-            g = Mq + (long)(r0 + 8 * blk + rl) * ld + c0 + 2 * (cs ^ rl);
-        } else {   // k rows r0 + 2 blk, +1; complex columns c0 .. c0+63
-            const int kl = lane >> 5, cs = lane & 31;
-            g = Mq + (long)(r0 + 2 * blk + kl) * ld + c0 + 2 * cs;
+    for (int j = 0; j < (NBLK + NW - 1) / NW; ++j) {
+        const int blk = j * NW + wave;  // 1 KB block of the tile
+        if (blk < NBLK) {
+            const float2 *g;
+            if (KC) {  // rows r0 + 8 blk .. +7, complex k c0 .. c0+15
+                const int rl = lane >> 3, cs = lane & 7;
+                g = Mq + (long)(r0 + 8 * blk + rl) * ld + c0 + 2 * (cs ^ rl);
+            } else {   // 16-byte chunk c of the tile stored as it lies: k row c / (ROWS/2), complex columns 2 (c % (ROWS/2))
+                const int c = blk * 64 + lane;
+                const int kl = c / (ROWS / 2), cs = c % (ROWS / 2);
+                g = Mq + (long)(r0 + kl) * ld + c0 + 2 * cs;
+            }
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1))) *)g,
+                (void __attribute__((address_space(3))) *)(lds + blk * 256), 16, 0, 0);
         }
-        __builtin_amdgcn_global_load_lds(
-            (const void __attribute__((address_space(1))) *)g,
-            (void __attribute__((address_space(3))) *)(lds + blk * 256), 16, 0, 0);
     }
 }
 
-// One 64x64 tile, workgroup index wg = frequency * tiles + tile.  lds: 4 operand tiles of 8 KB
-// (A and B, double-buffered).
-template <int MODE>
+// One 64 x (32 WN) tile by 2 x WN waves, workgroup index wg = frequency * tiles + tile.
+// lds: A tiles (8 KB) and B tiles (4 WN KB), double-buffered.
+template <int MODE, int WN>
 __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restrict__ A,
                                                const float2 *__restrict__ B, float2 *__restrict__ C,
                                                int M, int N, int K, float alpha, int accumulate,
@@ -248,21 +254,25 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
 {
     constexpr bool A_KC = (MODE != 2);
     constexpr bool B_KC = (MODE == 0);
-    constexpr int TILE = 64 * KT * 2;  // floats per operand tile (8 KB)
-    // buffer b of A at lds + b * TILE, of B at lds + (2 + b) * TILE
+    constexpr int BNW = 32 * WN;           // tile columns
+    constexpr int NW = 2 * WN;             // waves
+    constexpr int TILE = 64 * KT * 2;      // floats per A tile (8 KB)
+    constexpr int TILEB = BNW * KT * 2;    // floats per B tile
+    constexpr int LDB = 2 * BNW;           // floats per k row of a row-contiguous B tile
+    // buffer b of A at lds + b * TILE, of B at lds + 2 * TILE + b * TILEB
 
     const int tiles = tilesM * tilesN;
     const int q = wg / tiles;
     const int tile = wg - q * tiles;
     const int m0 = (tile / tilesN) * BM;
-    const int n0 = (tile % tilesN) * BN;
+    const int n0 = (tile % tilesN) * BNW;
     const float2 *Aq = A + (long)q * M * K;
     const float2 *Bq = B + (long)q * N * K;
     float2 *Cq = C + (long)q * M * N;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, h = lane >> 5;
 
     floatx16 cre, cim;
@@ -272,11 +282,11 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
     const int nk = K / KT;
     auto issue = [&](int kt, int buf) {
         const int k0 = kt * KT;
-        float *ab = lds + buf * TILE, *bb = lds + (2 + buf) * TILE;
-        if (A_KC) lds_direct_tile<true>(Aq, K, m0, k0, ab, wave, lane);   // A[m][k]
-        else      lds_direct_tile<false>(Aq, M, k0, m0, ab, wave, lane);  // A[k][m]
-        if (B_KC) lds_direct_tile<true>(Bq, K, n0, k0, bb, wave, lane);   // B[n][k]
-        else      lds_direct_tile<false>(Bq, N, k0, n0, bb, wave, lane);  // B[k][n]
+        float *ab = lds + buf * TILE, *bb = lds + 2 * TILE + buf * TILEB;
+        if (A_KC) lds_direct_tile<true, 64, NW>(Aq, K, m0, k0, ab, wave, lane);    // A[m][k]
+        else      lds_direct_tile<false, 64, NW>(Aq, M, k0, m0, ab, wave, lane);   // A[k][m]
+        if (B_KC) lds_direct_tile<true, BNW, NW>(Bq, K, n0, k0, bb, wave, lane);   // B[n][k]
+        else      lds_direct_tile<false, BNW, NW>(Bq, N, k0, n0, bb, wave, lane);  // B[k][n]
     };
 
     issue(0, 0);
@@ -293,7 +303,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
         if (kt + 1 < nk) issue(kt + 1, buf ^ 1);  // asynchronous: lands while this tile is multiplied
 
         const float *as = lds + buf * TILE;
-        const float *bs = lds + (2 + buf) * TILE;
+        const float *bs = lds + 2 * TILE + buf * TILEB;
         if (MODE == 0) {
             float a[16], b[16];
 #pragma unroll
@@ -319,7 +329,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
             }
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) {
-                const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDM + 2 * bcol);
+                const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDB + 2 * bcol);
                 cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.x, cre, 0, 0, 0);
                 cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.y, cim, 0, 0, 0);
                 cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], -vb.y, cre, 0, 0, 0);
@@ -330,7 +340,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
             for (int kk = 0; kk < 8; ++kk) {
                 // half-wave h owns k = 8h + kk: both components of conj(A)[k][arow] and B[k][bcol]
                 const float2 va = *reinterpret_cast<const float2 *>(as + (8 * h + kk) * LDM + 2 * arow);
-                const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDM + 2 * bcol);
+                const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDB + 2 * bcol);
                 cre = __builtin_amdgcn_mfma_f32_32x32x2f32(va.x, vb.x, cre, 0, 0, 0);
                 cim = __builtin_amdgcn_mfma_f32_32x32x2f32(va.x, vb.y, cim, 0, 0, 0);
                 cre = __builtin_amdgcn_mfma_f32_32x32x2f32(va.y, vb.y, cre, 0, 0, 0);
@@ -358,20 +368,22 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
     }
 }
 
-constexpr int LDSDIRECT_FLOATS = 4 * 64 * KT * 2;  // 32 KB
+constexpr int ldsdirect_floats(int wn) { return 2 * (64 * KT * 2 + 32 * wn * KT * 2); }
+constexpr int LDSDIRECT_FLOATS = ldsdirect_floats(2);  // 32 KB
 
-template <int MODE>
-__global__ __launch_bounds__(256) void cgemm_ldsdirect_kernel(const float2 *__restrict__ A,
-                                                              const float2 *__restrict__ B,
-                                                              float2 *__restrict__ C, int M, int N,
-                                                              int K, float alpha, int accumulate,
-                                                              int tilesM, int tilesN, int total_wgs,
-                                                              int chunk)
+// WN = 2: 64x64 tiles, 256 lanes.  WN = 3: 64x96 tiles, 384 lanes (N a multiple of 96 but not of 64).
+template <int MODE, int WN>
+__global__ __launch_bounds__(128 * WN) void cgemm_ldsdirect_kernel(const float2 *__restrict__ A,
+                                                                  const float2 *__restrict__ B,
+                                                                  float2 *__restrict__ C, int M, int N,
+                                                                  int K, float alpha, int accumulate,
+                                                                  int tilesM, int tilesN, int total_wgs,
+                                                                  int chunk)
 {
-    __shared__ __align__(16) float lds[LDSDIRECT_FLOATS];
+    __shared__ __align__(16) float lds[ldsdirect_floats(WN)];
     const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
     if (wg >= total_wgs) return;
-    ldsdirect_body<MODE>(lds, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, wg);
+    ldsdirect_body<MODE, WN>(lds, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, wg);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -594,7 +606,7 @@ __global__ __launch_bounds__(256) void cgemm_hybrid_kernel(const float2 *__restr
     if (j < chunk_direct) {
         const int wg = x * chunk_direct + j;
         if (wg >= direct_wgs) return;
-        ldsdirect_body<MODE>(lds, A, B, C, M, N, K, alpha, accumulate, M / 64, N / 64, wg);
+        ldsdirect_body<MODE, 2>(lds, A, B, C, M, N, K, alpha, accumulate, M / 64, N / 64, wg);
     } else {
         const int wg = x * chunk_split + (j - chunk_direct);
         if (wg >= split_wgs) return;
@@ -668,6 +680,19 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
             return hipGetLastError();
         }
     }
+    // N a multiple of 96 but not of 64 (config 5: 96 input planes): 64x96 tiles by six waves.  Measured
+    // at 2112 frequencies: 256x96x64 conj(A)^T B 293 us against 321 for the register-fed kernel, but
+    // 64x96x256 A B 290 against 279, so the plain product keeps the register-fed kernel.
+    if ((MODE != 1 || force == 8) && (m % 64) == 0 && (n % 96) == 0 && (n % 64) != 0 && (k % 16) == 0 && aligned16 &&
+        (force == 8 || (force < 0 && (long)n_freq * (m / 64) * (n / 96) >= 4 * 256))) {
+        const int t96 = n / 96;
+        const long tot = (long)n_freq * tilesM * t96;
+        const int ch = (int)((tot + 7) / 8);
+        hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 3>), dim3((unsigned)(ch * 8)), dim3(384), 0, s,
+                           reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
+                           reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, t96, (int)tot, ch);
+        return hipGetLastError();
+    }
     const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && total >= 4 * 256));
     if (!prefer_direct && (m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 &&
         tot32 * 4 < 0x7fffff00L) {
@@ -682,7 +707,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
     }
     const int chunk = (int)((total + 7) / 8);
     if (direct_ok && force != 0) {
-        hipLaunchKernelGGL(cgemm_ldsdirect_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
+        hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 2>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                            reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                            reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
                            (int)total, chunk);
