@@ -40,6 +40,9 @@ def stage_model(cfg, pass_, n, q):
     once written and once read; no scratch traffic)."""
     B, P, F, H, k, pad = cfg[:6]
     o = H + 2 * pad - k + 1
+    # the passes leave out the n - 2 frequencies that are conjugates of others (columns kx = 0 and
+    # n/2, rows above n/2): they are neither written, contracted nor read
+    q = q - (n - 2)
     fft = lambda planes, h: 4 * planes * h * h + 8 * planes * q
     mm_bytes = lambda m, nn_, kk: 8 * q * (m * kk + kk * nn_ + m * nn_)
     mm_flops = lambda m, nn_, kk: 8 * q * m * nn_ * kk
@@ -193,7 +196,7 @@ def measure_config(nn, torch, synth, name, steps, warmup):
             else:
                 ach = spec[1] / (ms_s * 1e-3) / 1e12
                 mnk = {"fprop": (B, F, P), "bprop": (B, P, F), "accgrad": (F, P, B)}[p]
-                entry["stages"][s] = {"kernel": mm_kernel_name(p, q, *mnk), "ms": ms_s, "bound": "mfma",
+                entry["stages"][s] = {"kernel": mm_kernel_name(p, q - (n - 2), *mnk), "ms": ms_s, "bound": "mfma",
                                       "flops": spec[1], "bytes": spec[2], "achieved": ach,
                                       "unit": "TFLOP/s", "peak": MFMA_FP32_PEAK_TF,
                                       "frac": ach / MFMA_FP32_PEAK_TF,

@@ -403,7 +403,7 @@ int fbfc_plan_stage_ms(const fbfc_plan *p, float *ms, int n)
 static fbfc::FwdArgs weight_args(const fbfc_plan *p, const float *weight)
 {
     const fbfc_conv_desc &d = p->d;
-    return fbfc::FwdArgs{weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w, 0, 0, {}};
+    return fbfc::FwdArgs{weight, p->w_freq, (long)d.out_planes * d.in_planes, d.k_h, d.k_w, 0, 0, {}, 1};
 }
 
 int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, const float *bias,
@@ -414,10 +414,14 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     hipStream_t s = static_cast<hipStream_t>(stream);
     const fbfc_conv_desc &d = p->d;
     const pass_geom &g = p->fprop;
-    const int N = p->info.fft_size, Q = p->info.n_freq;
+    const int N = p->info.fft_size;
+    // the contraction leaves out the frequencies that are conjugates of others (Hermitian symmetry
+    // along ky in the columns kx = 0 and N/2); the inverse transform does not read them
+    const int QH = fbfc::hermitian_count(N);
+    const fbfc::FreqMap fm = fbfc::hermitian_map(N);
     StageTimer tm(p, s);
     const fbfc::FwdArgs fin = {input, p->in_freq, (long)g.vbatch * d.in_planes, g.a_h, g.a_w, g.a_pad_u,
-                               g.a_pad_l, g.a_win};
+                               g.a_pad_l, g.a_win, 1};
     const fbfc::FwdArgs fw = weight_args(p, weight);
     if (!p->timed) {  // both forward FFTs in one launch; timed plans keep them apart to time each
         FBFC_TRY(fbfc::launch_rfft2d_pair(N, fin, fw, s), "rfft2d(input, weight)");
@@ -432,7 +436,7 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     float *res = p->reuse ? p->res_freq : p->out_freq;
     if (!p->reuse) p->have_out = false;
     // O[b][f] = 1/N^2 sum_p I[b][p] conj(W[f][p])   (SpatialConvolutionFBFFT.lua:157-164)
-    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(0, p->in_freq, p->w_freq, res, Q, g.vbatch, d.out_planes,
+    FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(0, p->in_freq, p->w_freq, res, QH, fm, g.vbatch, d.out_planes,
                                      d.in_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(fprop)");
     tm.done(FBFC_STAGE_MM);
     const fbfc::InvArgs inv = {res, output, (long)g.vbatch * d.out_planes, g.r_h, g.r_w, g.r_pad_u, g.r_pad_l,
@@ -450,10 +454,14 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     hipStream_t s = static_cast<hipStream_t>(stream);
     const fbfc_conv_desc &d = p->d;
     const pass_geom &g = p->bprop;
-    const int N = p->info.fft_size, Q = p->info.n_freq;
+    const int N = p->info.fft_size;
+    // the contraction leaves out the frequencies that are conjugates of others (Hermitian symmetry
+    // along ky in the columns kx = 0 and N/2); the inverse transform does not read them
+    const int QH = fbfc::hermitian_count(N);
+    const fbfc::FreqMap fm = fbfc::hermitian_map(N);
     StageTimer tm(p, s);
     const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)g.vbatch * d.out_planes, g.a_h, g.a_w,
-                               g.a_pad_u, g.a_pad_l, g.a_win};
+                               g.a_pad_u, g.a_pad_l, g.a_win, 1};
     const fbfc::FwdArgs fw = weight_args(p, weight);
     const bool need_w = !((p->reuse & FBFC_REUSE_WEIGHT) && p->have_w);
     if (!p->timed && need_w) {
@@ -472,7 +480,7 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     float *res = p->reuse ? p->res_freq : p->in_freq;
     if (!p->reuse) p->have_in = false;
     // GI[b][p] = 1/N^2 sum_f GO[b][f] W[f][p]   (SpatialConvolutionFBFFT.lua:244-251)
-    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(1, p->out_freq, p->w_freq, res, Q, g.vbatch, d.in_planes,
+    FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(1, p->out_freq, p->w_freq, res, QH, fm, g.vbatch, d.in_planes,
                                      d.out_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(bprop)");
     tm.done(FBFC_STAGE_MM);
     const fbfc::InvArgs inv = {res, grad_input, (long)g.vbatch * d.in_planes, g.r_h, g.r_w, g.r_pad_u,
@@ -490,12 +498,16 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     hipStream_t s = static_cast<hipStream_t>(stream);
     const fbfc_conv_desc &d = p->d;
     const pass_geom &g = p->accgrad;
-    const int N = p->info.fft_size, Q = p->info.n_freq;
+    const int N = p->info.fft_size;
+    // the contraction leaves out the frequencies that are conjugates of others (Hermitian symmetry
+    // along ky in the columns kx = 0 and N/2); the inverse transform does not read them
+    const int QH = fbfc::hermitian_count(N);
+    const fbfc::FreqMap fm = fbfc::hermitian_map(N);
     StageTimer tm(p, s);
     const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)g.vbatch * d.out_planes, g.g_h, g.g_w, 0, 0,
-                               g.g_win};
+                               g.g_win, 1};
     const fbfc::FwdArgs fin = {input, p->in_freq, (long)g.vbatch * d.in_planes, g.a_h, g.a_w, g.a_pad_u,
-                               g.a_pad_l, g.a_win};
+                               g.a_pad_l, g.a_win, 1};
     const bool need_go = !((p->reuse & FBFC_REUSE_OUTPUT) && p->have_out);
     const bool need_in = !((p->reuse & FBFC_REUSE_INPUT) && p->have_in);
     if (!p->timed && need_go && need_in) {
@@ -522,7 +534,7 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     float *res = p->reuse ? p->res_freq : p->w_freq;
     if (!p->reuse) p->have_w = false;
     // GW[f][p] = scale/N^2 sum_b conj(GO[b][f]) I[b][p]   (SpatialConvolutionFBFFT.lua:337-344)
-    FBFC_STAGE(tm, fbfc::launch_cgemm_freq(2, p->out_freq, p->in_freq, res, Q, d.out_planes, d.in_planes,
+    FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(2, p->out_freq, p->in_freq, res, QH, fm, d.out_planes, d.in_planes,
                                      g.vbatch, scale / ((float)N * (float)N), 0, s), "cgemm(accGrad)");
     tm.done(FBFC_STAGE_MM);
     fbfc::InvArgs inv = {res, grad_weight, (long)d.out_planes * d.in_planes, g.r_h, g.r_w, 0, 0, nullptr, 1, {},

@@ -28,6 +28,14 @@ namespace fbfc {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+__device__ __forceinline__ int map_freq(int i, const FreqMap &fm)
+{
+    if (fm.split == 0 || i < fm.split) return i;
+    const int j = i - fm.split;
+    const int row = j / fm.rowlen;
+    return fm.split + row * fm.nh + (j - row * fm.rowlen) + 1;
+}
+
 constexpr int BM = 64, BN = 64, KT = 16;
 constexpr int LDK = 2 * KT + 4;  // floats per row of a K-contiguous tile [64][KT] (+16 B pad)
 constexpr int LDM = 2 * 64;      // floats per row of a row-contiguous tile [KT][64]
@@ -70,7 +78,7 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
                                                          const float2 *__restrict__ B,
                                                          float2 *__restrict__ C, int M, int N, int K,
                                                          float alpha, int accumulate, int tilesM,
-                                                         int tilesN, int total_wgs, int chunk)
+                                                         int tilesN, int total_wgs, int chunk, FreqMap fm)
 {
     constexpr bool A_KC = (MODE != 2);
     constexpr bool B_KC = (MODE == 0);
@@ -83,8 +91,9 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
     const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
     if (wg >= total_wgs) return;
     const int tiles = tilesM * tilesN;
-    const int q = wg / tiles;
-    const int tile = wg - q * tiles;
+    const int qi = wg / tiles;
+    const int tile = wg - qi * tiles;
+    const int q = map_freq(qi, fm);
     const int m0 = (tile / tilesN) * BM;
     const int n0 = (tile % tilesN) * BN;
 
@@ -250,7 +259,7 @@ template <int MODE, int WN>
 __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restrict__ A,
                                                const float2 *__restrict__ B, float2 *__restrict__ C,
                                                int M, int N, int K, float alpha, int accumulate,
-                                               int tilesM, int tilesN, int wg)
+                                               int tilesM, int tilesN, int wg, int q_base, const FreqMap &fm)
 {
     constexpr bool A_KC = (MODE != 2);
     constexpr bool B_KC = (MODE == 0);
@@ -262,8 +271,9 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
     // buffer b of A at lds + b * TILE, of B at lds + 2 * TILE + b * TILEB
 
     const int tiles = tilesM * tilesN;
-    const int q = wg / tiles;
-    const int tile = wg - q * tiles;
+    const int qi = wg / tiles;
+    const int tile = wg - qi * tiles;
+    const int q = map_freq(q_base + qi, fm);
     const int m0 = (tile / tilesN) * BM;
     const int n0 = (tile % tilesN) * BNW;
     const float2 *Aq = A + (long)q * M * K;
@@ -378,12 +388,12 @@ __global__ __launch_bounds__(128 * WN) void cgemm_ldsdirect_kernel(const float2 
                                                                   float2 *__restrict__ C, int M, int N,
                                                                   int K, float alpha, int accumulate,
                                                                   int tilesM, int tilesN, int total_wgs,
-                                                                  int chunk)
+                                                                  int chunk, FreqMap fm)
 {
     __shared__ __align__(16) float lds[ldsdirect_floats(WN)];
     const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
     if (wg >= total_wgs) return;
-    ldsdirect_body<MODE, WN>(lds, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, wg);
+    ldsdirect_body<MODE, WN>(lds, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, wg, 0, fm);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -468,7 +478,7 @@ template <int MODE, int SK>
 __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *__restrict__ A,
                                             const float2 *__restrict__ B, float2 *__restrict__ C, int M,
                                             int N, int K, float alpha, int accumulate, int tilesM,
-                                            int tilesN, int total_tiles, int wg)
+                                            int tilesN, int total_tiles, int wg, int q_base, const FreqMap &fm)
 {
     constexpr int TPW = 4 / SK;  // 32x32 blocks per workgroup; SK waves share one block's K range
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -478,8 +488,9 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
     // consecutive blocks run along N: the waves of a workgroup share rows of A (through L1)
     const bool live = gtile < total_tiles;
     const int tiles = tilesM * tilesN;
-    const int q = live ? gtile / tiles : 0;
-    const int tile = live ? gtile - q * tiles : 0;
+    const int qi = live ? gtile / tiles : 0;
+    const int tile = live ? gtile - qi * tiles : 0;
+    const int q = map_freq(q_base + qi, fm);
     const int m0 = (tile / tilesN) * 32;
     const int n0 = (tile % tilesN) * 32;
     const float2 *Aq = A + (long)q * M * K;
@@ -577,12 +588,12 @@ __global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restr
                                                            float2 *__restrict__ C, int M, int N, int K,
                                                            float alpha, int accumulate, int tilesM,
                                                            int tilesN, int total_tiles, int total_wgs,
-                                                           int chunk)
+                                                           int chunk, FreqMap fm)
 {
     __shared__ float red[SK > 1 ? 4 : 1][32][64];
     const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
     if (wg >= total_wgs) return;
-    splitk_body<MODE, SK>(red, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, total_tiles, wg);
+    splitk_body<MODE, SK>(red, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, total_tiles, wg, 0, fm);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -598,7 +609,8 @@ __global__ __launch_bounds__(256) void cgemm_hybrid_kernel(const float2 *__restr
                                                            float2 *__restrict__ C, int M, int N, int K,
                                                            float alpha, int accumulate, int q_direct,
                                                            int direct_wgs, int chunk_direct,
-                                                           int split_tiles, int split_wgs, int chunk_split)
+                                                           int split_tiles, int split_wgs, int chunk_split,
+                                                           FreqMap fm)
 {
     __shared__ __align__(16) float lds[LDSDIRECT_FLOATS];
     static_assert(LDSDIRECT_FLOATS == 4 * 32 * 64, "both bodies share one buffer");
@@ -606,19 +618,19 @@ __global__ __launch_bounds__(256) void cgemm_hybrid_kernel(const float2 *__restr
     if (j < chunk_direct) {
         const int wg = x * chunk_direct + j;
         if (wg >= direct_wgs) return;
-        ldsdirect_body<MODE, 2>(lds, A, B, C, M, N, K, alpha, accumulate, M / 64, N / 64, wg);
+        ldsdirect_body<MODE, 2>(lds, A, B, C, M, N, K, alpha, accumulate, M / 64, N / 64, wg, 0, fm);
     } else {
         const int wg = x * chunk_split + (j - chunk_direct);
         if (wg >= split_wgs) return;
-        const long off = (long)q_direct;  // the split part starts at frequency q_direct
-        splitk_body<MODE, 4>(reinterpret_cast<float (*)[32][64]>(lds), A + off * M * K, B + off * N * K,
-                             C + off * M * N, M, N, K, alpha, accumulate, M / 32, N / 32, split_tiles, wg);
+        // the split part starts at frequency q_direct
+        splitk_body<MODE, 4>(reinterpret_cast<float (*)[32][64]>(lds), A, B, C, M, N, K, alpha, accumulate,
+                             M / 32, N / 32, split_tiles, wg, q_direct, fm);
     }
 }
 
 template <int MODE, int SK>
 static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_freq, int m, int n,
-                                int k, float alpha, int accumulate, hipStream_t s)
+                                int k, float alpha, int accumulate, FreqMap fm, hipStream_t s)
 {
     const int tm = m / 32, tn = n / 32;
     const long tot32 = (long)n_freq * tm * tn;
@@ -627,7 +639,7 @@ static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_
     hipLaunchKernelGGL((cgemm_splitk_kernel<MODE, SK>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                        reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tm, tn, (int)tot32,
-                       (int)wgs, chunk);
+                       (int)wgs, chunk, fm);
     return hipGetLastError();
 }
 
@@ -646,7 +658,7 @@ static int splitk_override()
 
 template <int MODE>
 static hipError_t launch_mode(const float *A, const float *B, float *C, int n_freq, int m, int n,
-                              int k, float alpha, int accumulate, hipStream_t s)
+                              int k, float alpha, int accumulate, FreqMap fm, hipStream_t s)
 {
     const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
     const long total = (long)n_freq * tilesM * tilesN;
@@ -676,7 +688,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
                                dim3(256), 0, s, reinterpret_cast<const float2 *>(A),
                                reinterpret_cast<const float2 *>(B), reinterpret_cast<float2 *>(C), m, n, k,
                                alpha, accumulate, q_direct, direct_wgs, chunk_direct, split_tiles,
-                               split_tiles, chunk_split);
+                               split_tiles, chunk_split, fm);
             return hipGetLastError();
         }
     }
@@ -690,7 +702,8 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
         const int ch = (int)((tot + 7) / 8);
         hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 3>), dim3((unsigned)(ch * 8)), dim3(384), 0, s,
                            reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
-                           reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, t96, (int)tot, ch);
+                           reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, t96, (int)tot, ch,
+                           fm);
         return hipGetLastError();
     }
     const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && total >= 4 * 256));
@@ -701,34 +714,40 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
         else if (tot32 < 4 * 1024 && (k % 64) == 0) sk = 4;
         else if (tot32 < 8 * 1024 && (k % 32) == 0) sk = 2;
         else sk = 1;
-        if (sk == 4 && (k % 64) == 0) return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
-        if (sk == 2 && (k % 32) == 0) return launch_splitk<MODE, 2>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
-        if (sk == 1) return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
+        if (sk == 4 && (k % 64) == 0) return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        if (sk == 2 && (k % 32) == 0) return launch_splitk<MODE, 2>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        if (sk == 1) return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
     }
     const int chunk = (int)((total + 7) / 8);
     if (direct_ok && force != 0) {
         hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 2>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                            reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                            reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
-                           (int)total, chunk);
+                           (int)total, chunk, fm);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                        reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
-                       (int)total, chunk);
+                       (int)total, chunk, fm);
     return hipGetLastError();
+}
+
+hipError_t launch_cgemm_freq_map(int mode, const float *A, const float *B, float *C, int n_freq, FreqMap fm,
+                                 int m, int n, int k, float alpha, int accumulate, hipStream_t s)
+{
+    switch (mode) {
+        case 0: return launch_mode<0>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        case 1: return launch_mode<1>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        case 2: return launch_mode<2>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_cgemm_freq(int mode, const float *A, const float *B, float *C, int n_freq, int m,
                              int n, int k, float alpha, int accumulate, hipStream_t s)
 {
-    switch (mode) {
-        case 0: return launch_mode<0>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
-        case 1: return launch_mode<1>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
-        case 2: return launch_mode<2>(A, B, C, n_freq, m, n, k, alpha, accumulate, s);
-        default: return hipErrorInvalidValue;
-    }
+    return launch_cgemm_freq_map(mode, A, B, C, n_freq, FreqMap{0, 1, 0}, m, n, k, alpha, accumulate, s);
 }
 
 }  // namespace fbfc

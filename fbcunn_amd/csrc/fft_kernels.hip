@@ -219,6 +219,7 @@ struct FwdJob {
     long planes;
     int h, w, padU, padL, vec4;
     int tbl_off;  // windowed operand: float offset of the window table in LDS
+    int herm;     // leave out the entries (ky > N/2, kx in {0, N/2}): conjugates of (N - ky, kx)
     Window win;
 };
 
@@ -239,6 +240,7 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
     const int h = second ? job1.h : job0.h, w = second ? job1.w : job0.w;
     const int padU = second ? job1.padU : job0.padU, padL = second ? job1.padL : job0.padL;
     const int vec4 = second ? job1.vec4 : job0.vec4;
+    const int herm = second ? job1.herm : job0.herm;
     const long x0 = plane_group<N>(blockIdx.x - (second ? blocks0 : 0u)) * T;
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
@@ -388,10 +390,13 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
                 constexpr int kn = (N - ky) % N;
                 const float zr = re[brev<N>(ky)], zi = im[brev<N>(ky)];
                 const float nr = re[brev<N>(kn)], ni = im[brev<N>(kn)];
-                *reinterpret_cast<float2 *>(obase + ky * rowbytes + voff) =
-                    make_float2(0.5f * (zr + nr), 0.5f * (zi - ni));
-                *reinterpret_cast<float2 *>(obase + ky * rowbytes + vnyq) =
-                    make_float2(0.5f * (zi + ni), 0.5f * (nr - zr));
+                // both columns are spectra of real sequences: rows above N/2 repeat rows below it
+                if (ky <= N / 2 || !herm) {
+                    *reinterpret_cast<float2 *>(obase + ky * rowbytes + voff) =
+                        make_float2(0.5f * (zr + nr), 0.5f * (zi - ni));
+                    *reinterpret_cast<float2 *>(obase + ky * rowbytes + vnyq) =
+                        make_float2(0.5f * (zi + ni), 0.5f * (nr - zr));
+                }
             });
         }
     }
@@ -451,13 +456,18 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void irfft2d_kernel(co
                 im[ky] = v.y;
             });
         } else {
-            // pack columns 0 and N/2 (each the spectrum of a real sequence): C = X0 + i XN
-            static_for<N>([&](auto kk) {
+            // pack columns 0 and N/2 (each the spectrum of a real sequence): C = X0 + i XN.  Rows
+            // above N/2 are the conjugates of the rows below it and are not read.
+            static_for<N / 2 + 1>([&](auto kk) {
                 constexpr int ky = decltype(kk)::value;
                 const float2 a = *reinterpret_cast<const float2 *>(ibase + ky * rowbytes + voff);
                 const float2 b = *reinterpret_cast<const float2 *>(ibase + ky * rowbytes + vnyq);
                 re[ky] = a.x - b.y;
                 im[ky] = a.y + b.x;
+                if constexpr (ky > 0 && ky < N / 2) {
+                    re[N - ky] = a.x + b.y;
+                    im[N - ky] = b.x - a.y;
+                }
             });
         }
         fft_inplace<N, true>(re, im);
@@ -583,6 +593,7 @@ static FwdJob make_job(const FwdArgs &a)
     j.h = a.h; j.w = a.w; j.padU = a.padU; j.padL = a.padL;
     j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::T * a.h * a.w) % 4 == 0);
     j.tbl_off = 0;
+    j.herm = a.herm;
     j.win = a.win;
     return j;
 }
@@ -692,7 +703,7 @@ static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStr
 hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                          int padL, hipStream_t s)
 {
-    const FwdArgs a = {in, out, planes, h, w, padU, padL, {}};
+    const FwdArgs a = {in, out, planes, h, w, padU, padL, {}, 0};
     return dispatch_fwd(N, a, nullptr, s);
 }
 

@@ -24,9 +24,12 @@ struct FwdArgs {
     long planes;  // virtual planes when windowed
     int h, w, padU, padL;
     Window win;
+    int herm;  // 1: do not write the entries (ky > N/2, kx in {0, N/2}), conjugates of (N - ky, kx)
 };
 hipError_t launch_rfft2d_pair(int N, const FwdArgs &a, const FwdArgs &b, hipStream_t s);
 hipError_t launch_rfft2d_one(int N, const FwdArgs &a, hipStream_t s);
+// The inverse never reads the entries (ky > N/2, kx in {0, N/2}): it takes them as the conjugates of
+// (N - ky, kx), which they are for the spectrum of a real plane.
 hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,
                           int padL, const float *bias, int bias_period, hipStream_t s);
 
@@ -60,6 +63,20 @@ hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s);
 // for each of n_freq frequencies; operands frequency-major, complex interleaved.
 hipError_t launch_cgemm_freq(int mode, const float *A, const float *B, float *C, int n_freq, int m,
                              int n, int k, float alpha, int accumulate, hipStream_t s);
+
+// Which frequencies a contraction visits.  The spectrum of a real plane is Hermitian also along ky
+// in the columns kx = 0 and kx = N/2: X[N-ky][kx] = conj X[ky][kx], so the entries (ky > N/2,
+// kx in {0, N/2}) carry nothing new.  With a map, the i-th frequency contracted is
+//   i < split: i;  else split + row * nh + col + 1  with (row, col) = divmod(i - split, rowlen),
+// i.e. rows ky <= N/2 whole and rows ky > N/2 without their first and last column.
+// split = 0: every frequency of the buffer in order.
+struct FreqMap {
+    int split, rowlen, nh;
+};
+inline FreqMap hermitian_map(int N) { return FreqMap{(N / 2 + 1) * (N / 2 + 1), N / 2 - 1, N / 2 + 1}; }
+inline int hermitian_count(int N) { return (N / 2 + 1) * (N / 2 + 1) + (N / 2 - 1) * (N / 2 - 1); }
+hipError_t launch_cgemm_freq_map(int mode, const float *A, const float *B, float *C, int n_freq, FreqMap fm,
+                                 int m, int n, int k, float alpha, int accumulate, hipStream_t s);
 
 // bias_kernels.hip ---------------------------------------------------------------
 hipError_t launch_bias_add(float *out, const float *bias, int batch, int planes, int hw,

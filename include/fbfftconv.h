@@ -156,7 +156,10 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
 /* Replaces FFTWrapper_ffti (same files): UNNORMALISED complex-to-real inverse;
  * writes real[plane][r][s] = y[r+pad_u][s+pad_l] for r<h, s<w of the N x N result.
  * If bias != NULL, bias[plane % bias_period] is added to every element of the
- * plane (the fused form of updateOutputBiasFFI, src/ConvolutionBias.cu:39-51). */
+ * plane (the fused form of updateOutputBiasFFI, src/ConvolutionBias.cu:39-51).
+ * As in any complex-to-real transform the input is taken to be the spectrum of a real
+ * plane: the entries (ky > N/2, kx in {0, N/2}) are not read but taken as the
+ * conjugates of (N - ky, kx). */
 int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l,
                 int fft_size, float *real, const float *bias, int bias_period, void *stream);
 
