@@ -65,12 +65,9 @@ def stage_model(cfg, pass_, n, q):
 # (profiles/hbm_traffic_all_configs.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, the
 # factors a 256 MiB device copy gives for the same counters (--calibrate-copy).
 MEASURED_TRAFFIC_MAIN = {
-    "cgemm_hybrid_kernel<0>": (18462 * 2.0 + 18432) * 1024,   # same operands and result as the
-    "cgemm_hybrid_kernel<1>": (18462 * 2.0 + 18432) * 1024,   # split-K kernel it replaced; to be
-    "cgemm_hybrid_kernel<2>": (18463 * 2.0 + 18432) * 1024,   # re-measured with the next counter run
-    "cgemm_splitk_kernel<0, 4>": (18462 * 2.0 + 18432) * 1024,
-    "cgemm_splitk_kernel<1, 4>": (18462 * 2.0 + 18432) * 1024,
-    "cgemm_splitk_kernel<2, 4>": (18463 * 2.0 + 18432) * 1024,
+    "cgemm_hybrid_kernel<0>": (17087 * 2.0 + 16640) * 1024,
+    "cgemm_hybrid_kernel<1>": (17088 * 2.0 + 16640) * 1024,
+    "cgemm_hybrid_kernel<2>": (17087 * 2.0 + 16640) * 1024,
 }
 
 KERNEL_OF_STAGE = {"fft_a": "rfft2d_kernel", "fft_b": "rfft2d_kernel", "mm": "cgemm_freq_kernel",
