@@ -54,6 +54,7 @@ SIGNATURES = {
     "fbfc_update_output": (_i, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "fbfc_update_grad_input": (_i, [_vp, _vp, _vp, _vp, _vp]),
     "fbfc_acc_grad_parameters": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _vp]),
+    "fbfc_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp]),
     "fbfc_plan_set_reuse": (_i, [_vp, ctypes.c_uint]),
     "fbfc_plan_set_timed": (_i, [_vp, _i]),
     "fbfc_plan_stage_ms": (_i, [_vp, ctypes.POINTER(_f), _i]),

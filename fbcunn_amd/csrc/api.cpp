@@ -490,8 +490,10 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     return tm.finish();
 }
 
-int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad_output,
-                             float *grad_weight, float *grad_bias, float scale, void *stream)
+// reuse_go: the spectrum of gradOutput that updateGradInput just left in the plan is taken as is
+static int acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad_output,
+                               float *grad_weight, float *grad_bias, float scale, bool reuse_go,
+                               void *stream)
 {
     if (p == nullptr || input == nullptr || grad_output == nullptr || grad_weight == nullptr)
         return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
@@ -508,7 +510,7 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
                                g.g_win, 1};
     const fbfc::FwdArgs fin = {input, p->in_freq, (long)g.vbatch * d.in_planes, g.a_h, g.a_w, g.a_pad_u,
                                g.a_pad_l, g.a_win, 1};
-    const bool need_go = !((p->reuse & FBFC_REUSE_OUTPUT) && p->have_out);
+    const bool need_go = !(((p->reuse & FBFC_REUSE_OUTPUT) || reuse_go) && p->have_out);
     const bool need_in = !((p->reuse & FBFC_REUSE_INPUT) && p->have_in);
     if (!p->timed && need_go && need_in) {
         FBFC_TRY(fbfc::launch_rfft2d_pair(N, fgo, fin, s), "rfft2d(gradOutput, input)");
@@ -551,6 +553,22 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     }
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();
+}
+
+int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad_output,
+                             float *grad_weight, float *grad_bias, float scale, void *stream)
+{
+    return acc_grad_parameters(p, input, grad_output, grad_weight, grad_bias, scale, false, stream);
+}
+
+int fbfc_backward(fbfc_plan *p, const float *input, const float *grad_output, const float *weight,
+                  float *grad_input, float *grad_weight, float *grad_bias, float scale, void *stream)
+{
+    const int rc = fbfc_update_grad_input(p, grad_output, weight, grad_input, stream);
+    if (rc != FBFC_OK) return rc;
+    // updateGradInput leaves FFT(gradOutput) in the plan (have_out; not for tiled plans, whose two
+    // passes window gradOutput differently)
+    return acc_grad_parameters(p, input, grad_output, grad_weight, grad_bias, scale, true, stream);
 }
 
 int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,

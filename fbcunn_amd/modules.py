@@ -201,8 +201,19 @@ class SpatialConvolutionFFT:
                                              ctypes.c_float(scale), _stream()))
 
     def backward(self, input, gradOutput, scale=1.0):
-        self.updateGradInput(input, gradOutput)
-        self.accGradParameters(input, gradOutput, scale)
+        """updateGradInput + accGradParameters sharing FFT(gradOutput)
+        (SpatialConvolutionFFT.lua:405-416)."""
+        self._check_input(input)
+        _check_tensor(gradOutput, "gradOutput", 4)
+        B, _, H, W = input.shape
+        plan = self._plan_for(B, H, W)
+        if tuple(gradOutput.shape) != (B, self.nOutputPlane, plan.info.out_h, plan.info.out_w):
+            raise ValueError("gradOutput has the wrong shape")
+        if self.gradInput is None or self.gradInput.shape != input.shape:
+            self.gradInput = torch.empty_like(input)
+        check(lib().fbfc_backward(plan.handle, _ptr(input), _ptr(gradOutput), _ptr(self.weight),
+                                  _ptr(self.gradInput), _ptr(self.gradWeight), _ptr(self.gradBias),
+                                  ctypes.c_float(scale), _stream()))
         return self.gradInput
 
     def cleanupBuffers(self):

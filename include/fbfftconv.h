@@ -121,6 +121,14 @@ int fbfc_update_grad_input(fbfc_plan *plan, const float *grad_output, const floa
 int fbfc_acc_grad_parameters(fbfc_plan *plan, const float *input, const float *grad_output,
                              float *grad_weight, float *grad_bias, float scale, void *stream);
 
+/* Replaces SpatialConvolutionFFT:backward (fbcunn/SpatialConvolutionFFT.lua:405-416):
+ * updateGradInput followed by accGradParameters, the second reusing the spectrum of
+ * gradOutput the first one computed (the reference passes its outputTransposeBuffer in the
+ * reuse list) whatever the plan's reuse policy.  Tiled plans recompute it (their two passes
+ * window gradOutput differently).  Results equal those of the two separate calls. */
+int fbfc_backward(fbfc_plan *plan, const float *input, const float *grad_output, const float *weight,
+                  float *grad_input, float *grad_weight, float *grad_bias, float scale, void *stream);
+
 /* Memory-reuse policy of the module (SpatialConvolutionFFT.lua:59-63,216-240;
  * used at SpatialConvolutionFBFFT.lua:226-230,305-322): with a flag set, the
  * pass that would recompute that spectrum reuses the one the previous pass left

@@ -205,3 +205,32 @@ def test_module_argument_errors(nn):
     with pytest.raises(nn.FbfcError) as e:
         net.updateOutput(torch.zeros(1, 3, 200, 200, device="cuda"))   # FFT size 256: beyond fbfft's 128
     assert e.value.code == 2
+
+
+@pytest.mark.parametrize("cls,extra", [("SpatialConvolutionFBFFT", ()), ("SpatialConvolutionFFTTiled", (16, 16))])
+def test_backward_equals_the_two_passes(nn, oracle, cls, extra):
+    """backward() shares FFT(gradOutput) between its two passes (SpatialConvolutionFFT.lua:405-416):
+    same results as updateGradInput + accGradParameters, and as the oracle."""
+    B, P, F, k, H, pad = 3, 5, 4, 3, 29, 1
+    x = synth.uniform(41, (B, P, H, H), stream=0)
+    w = synth.normal(41, (F, P, k, k), 0.0, 0.05, stream=1)
+    g = synth.uniform(41, (B, F, H, H), stream=3)
+    xd, gd = dev(x), dev(g)
+    a = getattr(nn, cls)(P, F, k, k, 1, 1, pad, pad, *extra)
+    b = getattr(nn, cls)(P, F, k, k, 1, 1, pad, pad, *extra)
+    for net in (a, b):
+        net.weight.copy_(dev(w))
+        net.gradWeight.fill_(float("nan"))
+        net.gradBias.fill_(float("nan"))
+    gin = host(a.backward(xd, gd, 0.7))
+    b.updateGradInput(xd, gd)
+    b.accGradParameters(xd, gd, 0.7)
+    assert np.array_equal(gin, host(b.gradInput))
+    assert np.array_equal(host(a.gradWeight), host(b.gradWeight))
+    assert np.array_equal(host(a.gradBias), host(b.gradBias))
+    p4 = (pad,) * 4
+    _close(gin, oracle.convolution_full(g, w, (1, 1), p4), "gradInput")
+    _close(host(a.gradWeight), oracle.cross_correlation_reverse_valid(x, g, (1, 1), 0.7, p4), "gradWeight")
+    _close(host(a.gradBias), oracle.bias_acc_grad_parameters(g, 0.7), "gradBias")
+    a.cleanupBuffers()
+    b.cleanupBuffers()
