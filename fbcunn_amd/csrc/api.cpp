@@ -87,6 +87,7 @@ int plan_query(const fbfc_conv_desc *d, fbfc_plan_info *info)
 void set_geometry(fbfc_plan *p, int tile_h, int tile_w);
 
 bool fft_size_ok(int n) { return n == 8 || n == 16 || n == 32 || n == 64 || n == 128; }
+bool fft_size_tiny(int n) { return n == 2 || n == 4; }
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
@@ -575,10 +576,16 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
                float *freq, void *stream)
 {
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
-    if (!fft_size_ok(fft_size)) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
+    if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
+        return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
     if (planes < 1 || h < 1 || w < 1 || pad_u < 0 || pad_l < 0 || h + pad_u > fft_size ||
         w + pad_l > fft_size)
         return fail(FBFC_ERR_INVALID_ARGUMENT, "plane plus padding must fit the FFT size");
+    if (fft_size_tiny(fft_size)) {
+        FBFC_TRY(fbfc::launch_rfft2d_tiny(fft_size, real, freq, planes, h, w, pad_u, pad_l,
+                                          static_cast<hipStream_t>(stream)), "rfft2d");
+        return FBFC_OK;
+    }
     FBFC_TRY(fbfc::launch_rfft2d(fft_size, real, freq, planes, h, w, pad_u, pad_l,
                                  static_cast<hipStream_t>(stream)), "rfft2d");
     return FBFC_OK;
@@ -588,13 +595,43 @@ int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad
                 float *real, const float *bias, int bias_period, void *stream)
 {
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
-    if (!fft_size_ok(fft_size)) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
+    if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
+        return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
     if (planes < 1 || h < 1 || w < 1 || pad_u < 0 || pad_l < 0 || h + pad_u > fft_size ||
         w + pad_l > fft_size)
         return fail(FBFC_ERR_INVALID_ARGUMENT, "plane plus padding must fit the FFT size");
     if (bias != nullptr && bias_period < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "bias_period must be positive");
+    if (fft_size_tiny(fft_size)) {
+        FBFC_TRY(fbfc::launch_irfft2d_tiny(fft_size, freq, real, planes, h, w, pad_u, pad_l, bias, bias_period,
+                                           static_cast<hipStream_t>(stream)), "irfft2d");
+        return FBFC_OK;
+    }
     FBFC_TRY(fbfc::launch_irfft2d(fft_size, freq, real, planes, h, w, pad_u, pad_l, bias, bias_period,
                                   static_cast<hipStream_t>(stream)), "irfft2d");
+    return FBFC_OK;
+}
+
+static bool fft1d_size_ok(int n) { return n >= 2 && n <= 128 && (n & (n - 1)) == 0; }
+
+int fbfc_fft1d(const float *real, long rows, int n, int pad_l, int fft_size, float *freq, void *stream)
+{
+    if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!fft1d_size_ok(fft_size)) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
+    if (rows < 1 || n < 1 || pad_l < 0 || n + pad_l > fft_size)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "row plus padding must fit the FFT size");
+    FBFC_TRY(fbfc::launch_rfft1d(fft_size, real, freq, rows, n, pad_l, static_cast<hipStream_t>(stream)),
+             "rfft1d");
+    return FBFC_OK;
+}
+
+int fbfc_ifft1d(const float *freq, long rows, int n, int pad_l, int fft_size, float *real, void *stream)
+{
+    if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!fft1d_size_ok(fft_size)) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
+    if (rows < 1 || n < 1 || pad_l < 0 || n + pad_l > fft_size)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "row plus padding must fit the FFT size");
+    FBFC_TRY(fbfc::launch_irfft1d(fft_size, freq, real, rows, n, pad_l, static_cast<hipStream_t>(stream)),
+             "irfft1d");
     return FBFC_OK;
 }
 

@@ -56,6 +56,17 @@ struct InvArgs {
 };
 hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s);
 
+// fft_small.hip ------------------------------------------------------------------
+// 1-D batched transforms, N in {2,4,...,128}: rows of n reals at pad_l of the N-point canvas
+// <-> (rows, N/2+1) complex, row-major; the inverse is unnormalised.
+hipError_t launch_rfft1d(int N, const float *in, float *out, long rows, int n, int pad_l, hipStream_t s);
+hipError_t launch_irfft1d(int N, const float *in, float *out, long rows, int n, int pad_l, hipStream_t s);
+// 2-D transforms of size 2 and 4 (frequency-major spectrum, as for the larger sizes)
+hipError_t launch_rfft2d_tiny(int N, const float *in, float *out, long planes, int h, int w, int pad_u,
+                              int pad_l, hipStream_t s);
+hipError_t launch_irfft2d_tiny(int N, const float *in, float *out, long planes, int h, int w, int pad_u,
+                               int pad_l, const float *bias, int bias_period, hipStream_t s);
+
 // cgemm_kernels.hip ------------------------------------------------------------
 // mode 0: C[m][n] (+)= alpha * sum_k A[m][k] * conj(B[n][k])   A (m x k), B (n x k)
 // mode 1: C[m][n] (+)= alpha * sum_k A[m][k] * B[k][n]         A (m x k), B (k x n)

@@ -271,19 +271,33 @@ class SpatialConvolutionFFTTiledIterated(SpatialConvolutionFFTTiled):
 class FFTWrapper:
     """nn.FFTWrapper with the fbfft backend (fbcunn/FFTWrapper.lua:53-132).
 
-    fft(time, frequency): time (..., h, w) real; frequency is frequency-major:
-    a float tensor of shape (N, N/2+1, planes, 2).  ffti is unnormalised."""
+    Two transform dimensions: time (..., h, w) real, frequency a float tensor of shape
+    (N, N/2+1, planes, 2), frequency-major.  One transform dimension: time (..., n) real,
+    frequency (rows, N/2+1, 2) as in the reference.  ffti is unnormalised.  With timed set,
+    every call is measured (1 skipped + 1 timed run, src/fft/FFTWrapperLua.cpp:106-134) and
+    `lastTiming` holds {"ms", "GNlogN/s"} computed like the reference's log line (:137-152)."""
 
     def __init__(self, cufft=None, padLeft=0, padUp=0, timed=False):
         if cufft not in (None, "fbfft", False, 0):
             raise ValueError("only the fbfft implementation exists in this build")
         self.padLeft, self.padUp = padLeft, padUp
-        self.timed = timed
+        self.timed = bool(timed)
+        self.lastTiming = None
 
     @staticmethod
     def _dims(time, frequency):
         _check_tensor(time, "time")
-        _check_tensor(frequency, "frequency", 4)
+        _check_tensor(frequency, "frequency")
+        if frequency.dim() == 3:                       # one transform dimension
+            rows, nh = frequency.size(0), frequency.size(1)
+            if frequency.size(2) != 2 or nh < 2:
+                raise ValueError("frequency must be (rows, N/2+1, 2)")
+            n = 2 * (nh - 1)
+            if time.numel() != rows * time.size(-1):
+                raise ValueError("time and frequency disagree on the number of rows")
+            return 1, n, rows, 1, time.size(-1)
+        if frequency.dim() != 4:
+            raise ValueError("frequency must be (rows, N/2+1, 2) or (N, N/2+1, planes, 2)")
         n = frequency.size(0)
         planes = frequency.size(2)
         if frequency.size(1) != n // 2 + 1 or frequency.size(3) != 2:
@@ -291,19 +305,41 @@ class FFTWrapper:
         h, w = time.size(-2), time.size(-1)
         if time.numel() != planes * h * w:
             raise ValueError("time and frequency disagree on the number of planes")
-        return n, planes, h, w
+        return 2, n, planes, h, w
+
+    def _run(self, call, dims, n, batches):
+        if not self.timed:
+            call()
+            return
+        call()                                           # skipped trial
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        call()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        size = float(batches) * (n ** dims) * (1.0 + dims * math.log(n))   # the reference's formula
+        self.lastTiming = {"ms": ms, "GNlogN/s": size / 1e9 / (ms * 1e-3) if ms > 0 else float("inf")}
 
     def fft(self, time, frequency, batchDims=None):
-        n, planes, h, w = self._dims(time, frequency)
-        check(lib().fbfc_fft2d(_ptr(time), planes, h, w, self.padUp, self.padLeft, n,
-                               _ptr(frequency), _stream()))
+        dims, n, planes, h, w = self._dims(time, frequency)
+        if dims == 1:
+            self._run(lambda: check(lib().fbfc_fft1d(_ptr(time), planes, w, self.padLeft, n, _ptr(frequency),
+                                                     _stream())), 1, n, planes)
+        else:
+            self._run(lambda: check(lib().fbfc_fft2d(_ptr(time), planes, h, w, self.padUp, self.padLeft, n,
+                                                     _ptr(frequency), _stream())), 2, n, planes)
         return frequency
 
     def ffti(self, time, frequency, batchDims=None, bias=None):
-        n, planes, h, w = self._dims(time, frequency)
-        period = bias.numel() if bias is not None else 1
-        check(lib().fbfc_ifft2d(_ptr(frequency), planes, h, w, self.padUp, self.padLeft, n,
-                                _ptr(time), _ptr(bias), period, _stream()))
+        dims, n, planes, h, w = self._dims(time, frequency)
+        if dims == 1:
+            self._run(lambda: check(lib().fbfc_ifft1d(_ptr(frequency), planes, w, self.padLeft, n, _ptr(time),
+                                                      _stream())), 1, n, planes)
+        else:
+            period = bias.numel() if bias is not None else 1
+            self._run(lambda: check(lib().fbfc_ifft2d(_ptr(frequency), planes, h, w, self.padUp, self.padLeft, n,
+                                                      _ptr(time), _ptr(bias), period, _stream())), 2, n, planes)
         return time
 
 

@@ -157,7 +157,8 @@ int fbfc_plan_stage_ms(const fbfc_plan *plan, float *ms, int n);
  * Replaces FFTWrapper_fft with fbfft (src/fft/FFTWrapperLua.cpp:209-272 ->
  * fbfft2dHost, src/fft/FBFFTHost.cpp:39-116): batched 2-D real-to-complex FFT of
  * `planes` h x w planes, each implicitly zero-padded into an N x N canvas at
- * row pad_u, column pad_l.  N in {8,16,32,64,128}.  Output is frequency-major. */
+ * row pad_u, column pad_l.  N in {2,4,8,16,32,64,128} (the sizes the reference tests,
+ * test/test_FFTModule.lua:170-260).  Output is frequency-major. */
 int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l,
                int fft_size, float *freq, void *stream);
 
@@ -170,6 +171,14 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
  * conjugates of (N - ky, kx). */
 int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l,
                 int fft_size, float *real, const float *bias, int bias_period, void *stream);
+
+/* Replaces FFTWrapper_fft / FFTWrapper_ffti on tensors with ONE transform dimension
+ * (fbfft1dHost, src/fft/FBFFTHost.cpp:119-131): `rows` real sequences of n values, each
+ * zero-padded into fft_size points at pad_l, <-> freq (rows, fft_size/2+1, 2), row-major as in
+ * the reference.  fft_size in {2,4,...,128}; the inverse is unnormalised and writes
+ * real[row][i] = y[i + pad_l], i < n. */
+int fbfc_fft1d(const float *real, long rows, int n, int pad_l, int fft_size, float *freq, void *stream);
+int fbfc_ifft1d(const float *freq, long rows, int n, int pad_l, int fft_size, float *real, void *stream);
 
 /* Replaces transposeMMFFI (src/MM.cu:54-73): for each of n_freq frequencies,
  *   C (m x n) (=|+=) inv_norm * op(A) * op(B),   op = conjugate transpose if flagged.

@@ -27,6 +27,7 @@ def nn():
 
 CASES = [
     # N, planes, h, w, padU, padL
+    (2, 300, 2, 2, 0, 0), (2, 5, 1, 2, 1, 0), (4, 300, 4, 4, 0, 0), (4, 7, 3, 2, 1, 2),   # one lane per plane
     (8, 5, 8, 8, 0, 0), (8, 130, 3, 3, 0, 0), (8, 64, 5, 6, 2, 1),
     (16, 7, 13, 13, 1, 1), (16, 96, 16, 16, 0, 0), (16, 33, 3, 3, 0, 0), (16, 40, 10, 12, 3, 2),
     (32, 3, 27, 27, 2, 2), (32, 48, 32, 32, 0, 0), (32, 17, 5, 5, 0, 0), (32, 35, 20, 28, 5, 1),
@@ -140,3 +141,62 @@ def test_fft_argument_errors(nn):
     with pytest.raises(nn.FbfcError) as e:          # unsupported size, like fbfft's error code
         nn.FFTWrapper("fbfft").fft(x, torch.empty((24, 13, 4, 2), device="cuda"))
     assert e.value.code == 2
+
+
+# One transform dimension: the sizes and batch sizes of the reference's module test
+# (test/test_FFTModule.lua:170-193), plus padded rows.
+CASES_1D = [(n, rows, n, 0) for n in (2, 4, 8, 16, 32, 64, 128) for rows in (1, 127, 437)] + \
+           [(8, 33, 5, 2), (32, 1000, 27, 3), (128, 64, 100, 28), (16, 2, 1, 15)]
+
+
+@pytest.mark.parametrize("n,rows,m,pl", CASES_1D)
+def test_1d_forward_and_inverse(nn, oracle, n, rows, m, pl):
+    x = synth.uniform(300 + n + rows, (rows, m))
+    canvas = np.zeros((rows, n))
+    canvas[:, pl:pl + m] = x
+    want = np.fft.rfft(canvas)
+    freq = torch.full((rows, n // 2 + 1, 2), float("nan"), device="cuda")
+    w = nn.FFTWrapper("fbfft", pl, 0)
+    w.fft(dev(x), freq)
+    got = host(freq)
+    got = got[..., 0] + 1j * got[..., 1]
+    scale = max(np.abs(want).max(), 1e-30)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL * scale
+    # the oracle's naive DFT of the rows as 1 x n planes
+    pick = sorted({0, rows - 1})
+    o = oracle.dft2d_r2c(x[pick].reshape(len(pick), 1, m), 1, n, 0, pl)
+    assert np.abs(got[pick] - (o[..., 0] + 1j * o[..., 1]).reshape(len(pick), -1)).max() <= TOL * scale
+    # unnormalised inverse of an arbitrary real row's spectrum, read back at the padding offset
+    full = synth.uniform(400 + n + rows, (rows, n))
+    spec = np.fft.rfft(full.astype(np.float64))
+    fr = dev(np.stack([spec.real, spec.imag], -1).astype(np.float32))
+    out = torch.full((rows, m), float("nan"), device="cuda")
+    w.ffti(out, fr)
+    back = host(out)
+    wantb = full[:, pl:pl + m].astype(np.float64) * n
+    assert np.isfinite(back).all()
+    assert np.abs(back - wantb).max() <= 4 * TOL * np.abs(wantb).max()
+
+
+def test_1d_round_trip_and_timed_mode(nn):
+    n, rows = 64, 4096
+    x = synth.uniform(77, (rows, n))
+    freq = torch.empty((rows, n // 2 + 1, 2), device="cuda")
+    back = torch.empty((rows, n), device="cuda")
+    w = nn.FFTWrapper("fbfft", 0, 0, "timed")
+    w.fft(dev(x), freq)
+    assert w.lastTiming["ms"] > 0 and w.lastTiming["GNlogN/s"] > 0
+    w.ffti(back, freq)
+    assert np.abs(host(back) / n - x).max() <= 1e-5 * np.abs(x).max()
+
+
+def test_1d_errors(nn):
+    from fbcunn_amd._lib import FbfcError, ERR_UNSUPPORTED_SIZE, ERR_INVALID_ARGUMENT
+    w = nn.FFTWrapper("fbfft")
+    with pytest.raises(FbfcError) as e:
+        w.fft(torch.zeros(3, 256, device="cuda"), torch.zeros(3, 129, 2, device="cuda"))
+    assert e.value.code == ERR_UNSUPPORTED_SIZE
+    with pytest.raises(FbfcError) as e:
+        nn.FFTWrapper("fbfft", 5, 0).fft(torch.zeros(3, 6, device="cuda"), torch.zeros(3, 5, 2, device="cuda"))
+    assert e.value.code == ERR_INVALID_ARGUMENT
