@@ -23,6 +23,7 @@
 #include <cstdlib>
 
 #include "kernels.h"
+#include "store_nt.h"
 
 namespace fbfc {
 
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
                 v.x += o.x;
                 v.y += o.y;
             }
-            *dst = v;
+            store_nt(dst, v);
         }
     }
 }
@@ -374,7 +375,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
             v.x += o.x;
             v.y += o.y;
         }
-        *dst = v;
+        store_nt(dst, v);
     }
 }
 
@@ -547,7 +548,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
                 v.x += o.x;
                 v.y += o.y;
             }
-            *dst = v;
+            store_nt(dst, v);
         }
     } else {
         // add the SK partial accumulators of a block: each of its waves finalises 16/SK registers
@@ -577,7 +578,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
                 v.x += o.x;
                 v.y += o.y;
             }
-            *dst = v;
+            store_nt(dst, v);
         }
     }
 }
