@@ -46,19 +46,20 @@ def stage_model(cfg, pass_, n, q):
     fft = lambda planes, h: 4 * planes * h * h + 8 * planes * q
     mm_bytes = lambda m, nn_, kk: 8 * q * (m * kk + kk * nn_ + m * nn_)
     mm_flops = lambda m, nn_, kk: 8 * q * m * nn_ * kk
+    # "fft": both forward transforms of the pass, which are one launch; in accGradParameters the
+    # bias gradient (B*F complex numbers of FFT(gradOutput)'s zero-frequency row) rides on the
+    # inverse-FFT launch
     if pass_ == "fprop":
-        return {"fft_a": ("hbm", fft(B * P, H)), "fft_b": ("hbm", fft(F * P, k)),
+        return {"fft": ("hbm", fft(B * P, H) + fft(F * P, k)),
                 "mm": ("mfma", mm_flops(B, F, P), mm_bytes(B, F, P)),
                 "ifft": ("hbm", fft(B * F, o))}
     if pass_ == "bprop":
-        return {"fft_a": ("hbm", fft(B * F, o)), "fft_b": ("hbm", fft(F * P, k)),
+        return {"fft": ("hbm", fft(B * F, o) + fft(F * P, k)),
                 "mm": ("mfma", mm_flops(B, P, F), mm_bytes(B, P, F)),
                 "ifft": ("hbm", fft(B * P, H))}
-    # the bias gradient is read off the zero-frequency row of FFT(gradOutput): B*F complex numbers
-    return {"bias_grad": ("hbm", 8 * B * F),
-            "fft_a": ("hbm", fft(B * F, o)), "fft_b": ("hbm", fft(B * P, H)),
+    return {"fft": ("hbm", fft(B * F, o) + fft(B * P, H)),
             "mm": ("mfma", mm_flops(F, P, B), mm_bytes(F, P, B)),
-            "ifft": ("hbm", fft(F * P, k))}
+            "ifft": ("hbm", fft(F * P, k) + 8 * B * F)}
 
 
 # HBM bytes per launch at the main workload, from the committed rocprofv3 --pmc runs
@@ -70,8 +71,7 @@ MEASURED_TRAFFIC_MAIN = {
     "cgemm_hybrid_kernel<2>": (17087 * 2.0 + 16640) * 1024,
 }
 
-KERNEL_OF_STAGE = {"fft_a": "rfft2d_kernel", "fft_b": "rfft2d_kernel", "mm": "cgemm_freq_kernel",
-                   "ifft": "irfft2d_kernel", "bias_grad": "bias_grad_dc_kernel"}
+KERNEL_OF_STAGE = {"fft": "rfft2d_kernel", "mm": "cgemm_freq_kernel", "ifft": "irfft2d_kernel"}
 
 
 def mm_kernel_name(pass_, q, m, n, k):
@@ -178,6 +178,7 @@ def measure_config(nn, torch, synth, name, steps, warmup):
         for _ in range(reps):
             run_pass(net, x, g, p)
             for s, v in net.stageTimes(x).items():
+                s = "fft" if s in ("fft_a", "fft_b") else s   # one launch for both operands
                 acc[s] = acc.get(s, 0.0) + v
         net.timed = False
         model = stage_model(cfg, p, n, q)

@@ -424,14 +424,9 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     const fbfc::FwdArgs fin = {input, p->in_freq, (long)g.vbatch * d.in_planes, g.a_h, g.a_w, g.a_pad_u,
                                g.a_pad_l, g.a_win, 1};
     const fbfc::FwdArgs fw = weight_args(p, weight);
-    if (!p->timed) {  // both forward FFTs in one launch; timed plans keep them apart to time each
-        FBFC_TRY(fbfc::launch_rfft2d_pair(N, fin, fw, s), "rfft2d(input, weight)");
-    } else {
-        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fin, s), "rfft2d(input)");
-        tm.done(FBFC_STAGE_FFT_A);
-        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fw, s), "rfft2d(weight)");
-        tm.done(FBFC_STAGE_FFT_B);
-    }
+    // both forward FFTs in one launch
+    FBFC_STAGE(tm, fbfc::launch_rfft2d_pair(N, fin, fw, s), "rfft2d(input, weight)");
+    tm.done(FBFC_STAGE_FFT_A);
     p->have_in = true;
     p->have_w = true;
     float *res = p->reuse ? p->res_freq : p->out_freq;
@@ -465,16 +460,12 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
                                g.a_pad_u, g.a_pad_l, g.a_win, 1};
     const fbfc::FwdArgs fw = weight_args(p, weight);
     const bool need_w = !((p->reuse & FBFC_REUSE_WEIGHT) && p->have_w);
-    if (!p->timed && need_w) {
-        FBFC_TRY(fbfc::launch_rfft2d_pair(N, fgo, fw, s), "rfft2d(gradOutput, weight)");
+    if (need_w) {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_pair(N, fgo, fw, s), "rfft2d(gradOutput, weight)");
     } else {
         FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fgo, s), "rfft2d(gradOutput)");
-        tm.done(FBFC_STAGE_FFT_A);
-        if (need_w) {
-            FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fw, s), "rfft2d(weight)");
-            tm.done(FBFC_STAGE_FFT_B);
-        }
     }
+    tm.done(FBFC_STAGE_FFT_A);
     // a tiled updateGradInput transforms other windows of gradOutput than accGradParameters does
     p->have_out = !p->tiled;
     p->have_w = true;
@@ -513,27 +504,18 @@ static int acc_grad_parameters(fbfc_plan *p, const float *input, const float *gr
                                g.a_pad_l, g.a_win, 1};
     const bool need_go = !(((p->reuse & FBFC_REUSE_OUTPUT) || reuse_go) && p->have_out);
     const bool need_in = !((p->reuse & FBFC_REUSE_INPUT) && p->have_in);
-    if (!p->timed && need_go && need_in) {
-        FBFC_TRY(fbfc::launch_rfft2d_pair(N, fgo, fin, s), "rfft2d(gradOutput, input)");
-    } else {
-        if (need_go) {
-            FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fgo, s), "rfft2d(gradOutput)");
-            tm.done(FBFC_STAGE_FFT_A);
-        }
-        if (need_in) {
-            FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fin, s), "rfft2d(input)");
-            tm.done(FBFC_STAGE_FFT_B);
-        }
+    if (need_go && need_in) {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_pair(N, fgo, fin, s), "rfft2d(gradOutput, input)");
+        tm.done(FBFC_STAGE_FFT_A);
+    } else if (need_go) {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fgo, s), "rfft2d(gradOutput)");
+        tm.done(FBFC_STAGE_FFT_A);
+    } else if (need_in) {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fin, s), "rfft2d(input)");
+        tm.done(FBFC_STAGE_FFT_B);
     }
     p->have_out = true;
     p->have_in = true;
-    // gradBias[f] = scale * sum_b DC(gradOutput[b][f]) is read off the spectrum just computed:
-    // its own launch when timed, otherwise a few extra workgroups of the inverse-FFT launch.
-    if (grad_bias != nullptr && p->timed) {
-        FBFC_STAGE(tm, fbfc::launch_bias_grad_dc(p->out_freq, grad_bias, scale, g.vbatch, d.out_planes, s),
-                   "bias grad");
-        tm.done(FBFC_STAGE_BIAS_GRAD);
-    }
     float *res = p->reuse ? p->res_freq : p->w_freq;
     if (!p->reuse) p->have_w = false;
     // GW[f][p] = scale/N^2 sum_b conj(GO[b][f]) I[b][p]   (SpatialConvolutionFBFFT.lua:337-344)
@@ -542,16 +524,16 @@ static int acc_grad_parameters(fbfc_plan *p, const float *input, const float *gr
     tm.done(FBFC_STAGE_MM);
     fbfc::InvArgs inv = {res, grad_weight, (long)d.out_planes * d.in_planes, g.r_h, g.r_w, 0, 0, nullptr, 1, {},
                          nullptr, nullptr, 0.0f, 0, 0};
-    if (grad_bias != nullptr && !p->timed) {
+    if (grad_bias != nullptr) {
+        // gradBias[f] = scale * sum_b DC(gradOutput[b][f]) is read off the spectrum of gradOutput by a
+        // few extra workgroups of the inverse-FFT launch
         inv.go_freq = p->out_freq;
         inv.grad_bias = grad_bias;
         inv.scale = scale;
         inv.batch = g.vbatch;
         inv.out_planes = d.out_planes;
-        FBFC_TRY(fbfc::launch_irfft2d_args(N, inv, s), "irfft2d(gradWeight) + bias grad");
-    } else {
-        FBFC_STAGE(tm, fbfc::launch_irfft2d_args(N, inv, s), "irfft2d(gradWeight)");
     }
+    FBFC_STAGE(tm, fbfc::launch_irfft2d_args(N, inv, s), "irfft2d(gradWeight) + bias grad");
     tm.done(FBFC_STAGE_IFFT);
     return tm.finish();
 }

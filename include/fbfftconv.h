@@ -138,16 +138,18 @@ enum { FBFC_REUSE_NONE = 0, FBFC_REUSE_INPUT = 1, FBFC_REUSE_OUTPUT = 2, FBFC_RE
 int fbfc_plan_set_reuse(fbfc_plan *plan, unsigned flags);
 
 /* Per-stage timing, the counterpart of the `timed` flag of nn.FFTWrapper /
- * nn.CuBLASWrapper (src/fft/FFTWrapperLua.cpp:82-177): with reps > 0 each pass
- * launches every stage reps times back to back between two HIP events recorded
- * on the pass's stream (stages are pure functions of their inputs, so results
- * are unchanged) and synchronises at the end; fbfc_plan_stage_ms then reports
- * the mean time of one launch.  reps = 0 switches timing off.  Stage slots: */
-enum { FBFC_STAGE_FFT_A = 0,   /* first forward FFT of the pass  */
-       FBFC_STAGE_FFT_B = 1,   /* second forward FFT of the pass */
+ * nn.CuBLASWrapper (src/fft/FFTWrapperLua.cpp:82-177): with reps > 0 each pass issues
+ * every launch of its schedule reps times back to back between two HIP events recorded
+ * on the pass's stream (stages are pure functions of their inputs, so results are
+ * unchanged) and synchronises at the end; fbfc_plan_stage_ms then reports the mean time
+ * of one launch.  The launches are those of an untimed pass.  reps = 0 switches timing
+ * off.  Stage slots: */
+enum { FBFC_STAGE_FFT_A = 0,   /* the forward-FFT launch: both operands of the pass, or the
+                                  first one alone when the second is reused */
+       FBFC_STAGE_FFT_B = 1,   /* the second operand alone (when the first is reused) */
        FBFC_STAGE_MM = 2,      /* per-frequency contraction      */
-       FBFC_STAGE_IFFT = 3,    /* inverse FFT (+ bias)           */
-       FBFC_STAGE_BIAS_GRAD = 4,
+       FBFC_STAGE_IFFT = 3,    /* inverse FFT (+ bias, + bias gradient in accGradParameters) */
+       FBFC_STAGE_BIAS_GRAD = 4,  /* kept for layout; the bias gradient rides on the IFFT launch */
        FBFC_NUM_STAGES = 5 };
 int fbfc_plan_set_timed(fbfc_plan *plan, int reps);
 /* Milliseconds of each stage of the last timed pass (0 for a stage not run). */
