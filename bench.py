@@ -283,6 +283,23 @@ def measure_tiled(nn, torch, synth, steps, warmup):
     return out
 
 
+def measure_backward_step(nn, torch, synth, steps, warmup):
+    """The training step as a module user runs it: updateOutput, then backward(), whose two gradient
+    passes share FFT(gradOutput) (5 forward transforms per step instead of 6)."""
+    cfg = CONFIGS[MAIN]
+    B, P, F, H, k, pad = cfg[:6]
+    o = H + 2 * pad - k + 1
+    net, x, g = make_layer(nn, torch, synth, cfg)
+    def step():
+        net.updateOutput(x)
+        net.backward(x, g, 1.0)
+    ms = time_loop(torch, step, steps, warmup)
+    ms_b = time_loop(torch, lambda: net.backward(x, g, 1.0), steps, warmup)
+    net.cleanupBuffers()
+    return {"ms_per_step": ms, "ms_backward": ms_b,
+            "effective_tflops": 3 * 2.0 * B * F * P * o * o * k * k / (ms * 1e-3) / 1e12}
+
+
 def measure_copy_bandwidth(torch):
     """A plain 256 MiB device-to-device copy: what HBM delivers to a trivial kernel on this box."""
     a = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
@@ -392,6 +409,7 @@ def main():
         "stages": {k: v["stages"] for k, v in main_res["passes"].items()},
     }
     line["reuse_all_step"] = measure_reuse_step(nn, torch, synth, args.steps, args.warmup)
+    line["fprop_plus_backward_step"] = measure_backward_step(nn, torch, synth, args.steps, args.warmup)
     line["copy_256MiB"] = measure_copy_bandwidth(torch)
     if args.all_configs:
         others = {}

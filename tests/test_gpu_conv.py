@@ -234,3 +234,26 @@ def test_backward_equals_the_two_passes(nn, oracle, cls, extra):
     _close(host(a.gradBias), oracle.bias_acc_grad_parameters(g, 0.7), "gradBias")
     a.cleanupBuffers()
     b.cleanupBuffers()
+
+
+def test_backward_between_other_passes(nn, oracle):
+    """backward() reuses the spectrum updateGradInput leaves in the plan: with other passes and
+    changing inputs around it, every result must still be the one of the current inputs."""
+    B, P, F, k, H, pad = 4, 6, 5, 3, 13, 1
+    net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad)
+    w = synth.normal(51, (F, P, k, k), 0.0, 0.05, stream=1)
+    net.weight.copy_(dev(w))
+    net.bias.zero_()
+    p4 = (pad,) * 4
+    for it in range(4):
+        x = synth.uniform(60 + it, (B, P, H, H), stream=0)
+        g = synth.uniform(60 + it, (B, F, H, H), stream=3)
+        xd, gd = dev(x), dev(g)
+        out = net.updateOutput(xd)
+        gin = net.backward(xd, gd, 1.0)
+        out2 = net.updateOutput(xd)
+        _close(host(gin), oracle.convolution_full(g, w, (1, 1), p4), "gradInput %d" % it)
+        _close(host(net.gradWeight), oracle.cross_correlation_reverse_valid(x, g, (1, 1), 1.0, p4), "gradWeight %d" % it)
+        _close(host(net.gradBias), oracle.bias_acc_grad_parameters(g, 1.0), "gradBias %d" % it)
+        _close(host(out2), oracle.cross_correlation_valid(x, w, (1, 1), p4), "output %d" % it)
+    net.cleanupBuffers()
