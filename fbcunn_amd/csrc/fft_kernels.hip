@@ -30,20 +30,22 @@
 
 namespace fbfc {
 
-template <int N>
+template <int N, bool INVERSE = false>
 struct FftShape {
     static constexpr int T = 512 / N;       // planes per workgroup
     static constexpr int THREADS = 256;     // T * N / 2
     static constexpr int NH2 = N / 2;       // complex slots per tile row
     static constexpr int NH = N / 2 + 1;    // stored column frequencies
+    // (N = 32 forward: two phases halve the LDS footprint and a third workgroup fits a CU, measured
+    // 19.6 -> 17.4 us for config 3's pair of transforms; the inverse was slower that way and keeps one.)
     // Phases: the LDS tile holds NH2/PH of the tile columns at a time and the input /
     // output staging area T/PH planes at a time, so that two workgroups fit one CU's
     // 160 KB LDS even for N = 64 (a full 8-plane tile would need 117 KB).
-    static constexpr int PH = (N >= 128) ? 4 : (N >= 64) ? 2 : 1;
+    static constexpr int PH = (N >= 128) ? 4 : (N >= 64) ? 2 : (N == 32 && !INVERSE) ? 2 : 1;
     static constexpr int KXP = NH2 / PH;    // tile columns per phase
     static constexpr int TP = T / PH;       // planes per staging round
     // waves per SIMD the register budget is sized for (N = 128 keeps 256 values per lane)
-    static constexpr int MIN_WAVES = (N >= 128) ? 1 : PH;
+    static constexpr int MIN_WAVES = (N >= 128) ? 1 : (N == 32 && !INVERSE) ? 3 : PH;
     // padding (in complex elements) between tile rows: keeps the T-lane groups
     // of one wave on different LDS banks when T*8 bytes is below 128
     static constexpr int ROWPAD = (T * 8 < 128) ? (64 / 8) / 2 : 0;
@@ -418,14 +420,14 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
 // real[r][s] = y[r+padU][s+padL] (+ bias[plane % bias_period])
 // ---------------------------------------------------------------------------------
 template <int N, bool WIN>
-__global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void irfft2d_kernel(const float2 *__restrict__ in,
+__global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_kernel(const float2 *__restrict__ in,
                                                       float *__restrict__ out, long planes,
                                                       int h, int w, int padU, int padL,
                                                       const float *__restrict__ bias,
                                                       int bias_period, int vec4, BiasGradJob bgrad,
                                                       unsigned bgrad_blocks, Window win, int tbl_off)
 {
-    using S = FftShape<N>;
+    using S = FftShape<N, true>;
     constexpr int T = S::T;
     extern __shared__ __align__(16) float smem[];
     if (blockIdx.x < bgrad_blocks) {
@@ -572,13 +574,12 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void irfft2d_kernel(co
 // ---------------------------------------------------------------------------------
 // host launchers
 // ---------------------------------------------------------------------------------
-template <int N>
-static size_t fft_lds_bytes(int h, int w, int padU, bool inverse)
+template <int N, bool INVERSE>
+static size_t fft_lds_bytes(int h, int w, int padU)
 {
-    using S = FftShape<N>;
+    using S = FftShape<N, INVERSE>;
     const int y_lo = padU & ~1, y_hi = (padU + h + 1) & ~1;
     const size_t tile = (size_t)(y_hi - y_lo + 1) * S::ROWSTRIDE * sizeof(float2);
-    (void)inverse;
     (void)w;
     const size_t stage = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
     return ((tile > stage ? tile : stage) + 15) & ~(size_t)15;
@@ -627,13 +628,13 @@ static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    size_t lds = fft_lds_bytes<N>(a.h, a.w, a.padU, false);
+    size_t lds = fft_lds_bytes<N, false>(a.h, a.w, a.padU);
     const long blocks0 = fwd_blocks<N>(a.planes);
     long blocks = blocks0;
     FwdJob j0 = make_job<N>(a);
     FwdJob j1 = j0;
     if (second != nullptr) {
-        const size_t lds1 = fft_lds_bytes<N>(second->h, second->w, second->padU, false);
+        const size_t lds1 = fft_lds_bytes<N, false>(second->h, second->w, second->padU);
         if (lds1 > lds) lds = lds1;
         blocks += fwd_blocks<N>(second->planes);
         j1 = make_job<N>(*second);
@@ -651,7 +652,7 @@ static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_
 template <int N, bool WIN>
 static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
 {
-    using S = FftShape<N>;
+    using S = FftShape<N, true>;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&irfft2d_kernel<N, WIN>),
@@ -659,7 +660,7 @@ static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    size_t lds = fft_lds_bytes<N>(a.h, a.w, a.padU, true);
+    size_t lds = fft_lds_bytes<N, true>(a.h, a.w, a.padU);
     const int tbl_off = (int)(lds / sizeof(float));
     if (WIN) lds += S::T * sizeof(int4);
     long blocks = (a.planes + S::T - 1) / S::T;
