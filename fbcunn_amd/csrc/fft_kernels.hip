@@ -89,30 +89,58 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
         float4 *g4 = reinterpret_cast<float4 *>(g);
         int row = (tid * 4) / w, x = tid * 4 - row * w;
         const int drow = 1024 / w, dx = 1024 - drow * w;
-        for (int i = tid; i < n4; i += 256) {
-            float v[4];
-            if (TO_LDS) {
-                if constexpr (N >= 64) {
-                    // planes of this size add up to tensors no cache holds until their next use: stream
-                    // them (measured at 16384 planes of 55 x 55: 160 -> 136 us; smaller sizes got slower)
-                    const floatx4_nt q = __builtin_nontemporal_load(reinterpret_cast<const floatx4_nt *>(g4 + i));
-                    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
-                } else {
-                    const float4 q = g4[i];
-                    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        if constexpr (TO_LDS) {
+            // U loads in flight per lane before the first one is waited for: one load per round trip
+            // would leave the memory system idle for most of the copy
+            constexpr int U = (N >= 64) ? 12 : 8;
+            for (int i0 = tid; i0 < n4; i0 += 256 * U) {
+                float4 q[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int i = i0 + 256 * u;
+                    if (i < n4) {
+                        if constexpr (N >= 64) {
+                            // planes of this size add up to tensors no cache holds until their next use:
+                            // stream them (measured at 16384 planes of 55 x 55: 160 -> 136 us; smaller
+                            // sizes got slower)
+                            const floatx4_nt t = __builtin_nontemporal_load(reinterpret_cast<const floatx4_nt *>(g4 + i));
+                            q[u] = make_float4(t.x, t.y, t.z, t.w);
+                        } else {
+                            q[u] = g4[i];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int i = i0 + 256 * u;
+                    if (i < n4) {
+                        const float v[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+                        int r_ = row, x_ = x;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            smem[r_ * LDR + padL + x_] = v[c];
+                            if (++x_ == w) { x_ = 0; ++r_; }
+                        }
+                    }
+                    row += drow;
+                    x += dx;
+                    if (x >= w) { x -= w; ++row; }
                 }
             }
-            int r_ = row, x_ = x;
+        } else {
+            for (int i = tid; i < n4; i += 256) {
+                float v[4];
+                int r_ = row, x_ = x;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                float *sp = smem + r_ * LDR + padL + x_;
-                if (TO_LDS) *sp = v[c]; else v[c] = *sp;
-                if (++x_ == w) { x_ = 0; ++r_; }
+                for (int c = 0; c < 4; ++c) {
+                    v[c] = smem[r_ * LDR + padL + x_];
+                    if (++x_ == w) { x_ = 0; ++r_; }
+                }
+                store_nt(g4 + i, make_float4(v[0], v[1], v[2], v[3]));
+                row += drow;
+                x += dx;
+                if (x >= w) { x -= w; ++row; }
             }
-            if (!TO_LDS) store_nt(g4 + i, make_float4(v[0], v[1], v[2], v[3]));
-            row += drow;
-            x += dx;
-            if (x >= w) { x -= w; ++row; }
         }
         done = n4 << 2;
     }
@@ -138,6 +166,32 @@ __device__ __forceinline__ void store_freq(float2 *p, const float2 &v)
 {
     if constexpr (FftShape<N>::T * 8 >= 128) store_nt(p, v);
     else *p = v;
+}
+
+// Raw staging for the forward transform: the chunk of nfloats contiguous floats at g goes to LDS as it
+// lies, by LDS-direct loads (global_load_lds): no staging registers, no LDS store instructions and no
+// index arithmetic; the row pass then reads its rows at their (unaligned) places and masks the padding.
+// 16-byte pieces where the chunk allows (aligned16), 4-byte pieces for the rest.  The destination of a
+// wave instruction is wave-uniform; lane l lands at + l * size.
+__device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloats, bool aligned16, int tid)
+{
+    const int wave = tid >> 6, lane = tid & 63;
+    int done = 0;
+    if (aligned16) {
+        const int n16 = nfloats >> 2;
+        for (int p0 = wave * 64; p0 < n16; p0 += 256) {
+            if (p0 + lane < n16)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1))) *)(g + 4 * (p0 + lane)),
+                    (void __attribute__((address_space(3))) *)(raw + 4 * p0), 16, 0, 0);
+        }
+        done = n16 << 2;
+    }
+    for (int e0 = done + wave * 64; e0 < nfloats; e0 += 256) {
+        if (e0 + lane < nfloats)
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(g + e0 + lane),
+                                             (void __attribute__((address_space(3))) *)(raw + e0), 4, 0, 0);
+    }
 }
 
 // Zeroes the margins of nrows canvas rows and the all-zero row kept at index zrow.
@@ -245,7 +299,7 @@ struct FwdJob {
 
 // NZ < N: planes of at most NZ x NZ at the canvas origin (convolution kernels): the transforms skip
 // the inputs that are known to be zero.
-template <int N, bool WIN, int NZ>
+template <int N, bool WIN, int NZ, bool RAW>
 __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(FwdJob job0, FwdJob job1,
                                                                       unsigned blocks0)
 {
@@ -284,40 +338,70 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
     const bool vb = (ib >= 0) && (ib < h);
     const bool row_active = (t < np) && (va || vb);
 
-    // ---- stage the contiguous chunk of planes as zero-padded canvas rows, TP planes per round ----
+    // ---- stage the contiguous chunk of planes in LDS, TP planes per round ----
     constexpr int LDR = Canvas<N>::LDR;
-    const int zrow = S::TP * h;  // an all-zero row for canvas rows outside the plane
+    // Planes of odd height and width are staged raw, by asynchronous LDS-direct loads (their rows fall on
+    // different LDS banks by themselves); windowed operands, even sizes (a 32 x 32 plane staged raw puts
+    // every row on the same banks) and N = 128 (one-plane rounds need not be 16-byte multiples) are staged
+    // as zero-padded canvas rows.
+    static_assert(!RAW || (!WIN && N <= 64), "raw staging: plain operands, N <= 64");
+    const int zrow = S::TP * h;  // canvas staging: an all-zero row for canvas rows outside the plane
     static_for<S::PH>([&](auto hh) {
         constexpr int hs = decltype(hh)::value;
         int nph = np - hs * S::TP;
         nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
         if (hs > 0) __syncthreads();  // previous round fully read
-        bool windowed = false;
-        if constexpr (WIN) windowed = win.on != 0;
-        if (windowed) {
-            if (hs == 0) __syncthreads();  // window table complete
-            zero_canvas_margins<N>(smem, 0, w, 0, zrow, tid);  // the all-zero row only
-            copy_windows<N, true>(smem, const_cast<float *>(in), tbl, hs * S::TP, nph, h, w, 0, win, tid);
+        if constexpr (RAW) {
+            // N floats of slack in front: the first row is read from -padL on
+            float *raw = smem + N;
+            stage_raw(raw, in + (x0 + hs * S::TP) * hw, nph * hw, vec4 != 0, tid);
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's pieces have landed
+            __syncthreads();
+            if (row_active && (t / S::TP) == hs) {
+                const int tl = t - hs * S::TP;
+                const float *pa = raw + (va ? (tl * h + ia) * w : 0) - padL;
+                const float *pb = raw + (vb ? (tl * h + ib) * w : 0) - padL;
+                static_for<N>([&](auto xx) {
+                    constexpr int x = decltype(xx)::value;
+                    if constexpr (x < NZ) {
+                        const float a = pa[x], b = pb[x];
+                        const bool cx = (unsigned)(x - padL) < (unsigned)w;  // column inside the plane
+                        re[x] = (va && cx) ? a : 0.0f;
+                        im[x] = (vb && cx) ? b : 0.0f;
+                    } else {
+                        re[x] = 0.0f;
+                        im[x] = 0.0f;
+                    }
+                });
+            }
         } else {
-            zero_canvas_margins<N>(smem, nph * h, w, padL, zrow, tid);
-            copy_canvas<N, true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
-        }
-        __syncthreads();
-        if (row_active && (t / S::TP) == hs) {
-            const int tl = t - hs * S::TP;
-            const float4 *pa = reinterpret_cast<const float4 *>(smem + (va ? tl * h + ia : zrow) * LDR);
-            const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? tl * h + ib : zrow) * LDR);
-            static_for<N / 4>([&](auto jj) {
-                constexpr int j = decltype(jj)::value;
-                if constexpr (4 * j < NZ) {
-                    const float4 a = pa[j], b = pb[j];
-                    re[4 * j] = a.x; re[4 * j + 1] = a.y; re[4 * j + 2] = a.z; re[4 * j + 3] = a.w;
-                    im[4 * j] = b.x; im[4 * j + 1] = b.y; im[4 * j + 2] = b.z; im[4 * j + 3] = b.w;
-                } else {
-                    re[4 * j] = re[4 * j + 1] = re[4 * j + 2] = re[4 * j + 3] = 0.0f;
-                    im[4 * j] = im[4 * j + 1] = im[4 * j + 2] = im[4 * j + 3] = 0.0f;
-                }
-            });
+            bool windowed = false;
+            if constexpr (WIN) windowed = win.on != 0;
+            if (windowed) {
+                if (hs == 0) __syncthreads();  // window table complete
+                zero_canvas_margins<N>(smem, 0, w, 0, zrow, tid);  // the all-zero row only
+                copy_windows<N, true>(smem, const_cast<float *>(in), tbl, hs * S::TP, nph, h, w, 0, win, tid);
+            } else {
+                zero_canvas_margins<N>(smem, nph * h, w, padL, zrow, tid);
+                copy_canvas<N, true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
+            }
+            __syncthreads();
+            if (row_active && (t / S::TP) == hs) {
+                const int tl = t - hs * S::TP;
+                const float4 *pa = reinterpret_cast<const float4 *>(smem + (va ? tl * h + ia : zrow) * LDR);
+                const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? tl * h + ib : zrow) * LDR);
+                static_for<N / 4>([&](auto jj) {
+                    constexpr int j = decltype(jj)::value;
+                    if constexpr (4 * j < NZ) {
+                        const float4 a = pa[j], b = pb[j];
+                        re[4 * j] = a.x; re[4 * j + 1] = a.y; re[4 * j + 2] = a.z; re[4 * j + 3] = a.w;
+                        im[4 * j] = b.x; im[4 * j + 1] = b.y; im[4 * j + 2] = b.z; im[4 * j + 3] = b.w;
+                    } else {
+                        re[4 * j] = re[4 * j + 1] = re[4 * j + 2] = re[4 * j + 3] = 0.0f;
+                        im[4 * j] = im[4 * j + 1] = im[4 * j + 2] = im[4 * j + 3] = 0.0f;
+                    }
+                });
+            }
         }
     });
 
@@ -587,8 +671,11 @@ static size_t fft_lds_bytes(int h, int w, int padU)
     using S = FftShape<N, INVERSE>;
     const int y_lo = padU & ~1, y_hi = (padU + h + 1) & ~1;
     const size_t tile = (size_t)(y_hi - y_lo + 1) * S::ROWSTRIDE * sizeof(float2);
-    (void)w;
-    const size_t stage = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
+    // canvas-row staging (the inverse, windowed operands, N = 128) or, smaller, the raw chunk with N
+    // floats of slack on either side
+    const size_t canvas = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
+    const size_t raw = ((size_t)S::TP * h * w + 2 * N) * sizeof(float);
+    const size_t stage = canvas > raw ? canvas : raw;
     return ((tile > stage ? tile : stage) + 15) & ~(size_t)15;
 }
 
@@ -625,12 +712,15 @@ static bool window_ok(const Window &w, long planes, int h, int ww)
 }
 
 // second == nullptr: one tensor only
-template <int N, bool WIN, int NZ = N>
-static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
+// raw staging needs odd plane sizes (see the kernel) in every operand of the launch
+static bool raw_ok(const FwdArgs &a) { return (a.h & 1) && (a.w & 1) && !a.win.on; }
+
+template <int N, bool WIN, int NZ, bool RAW>
+static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
 {
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rfft2d_kernel<N, WIN, NZ>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rfft2d_kernel<N, WIN, NZ, RAW>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         attr_done = true;
@@ -651,9 +741,18 @@ static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_
         lds += FftShape<N>::T * sizeof(int4);
     }
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((rfft2d_kernel<N, WIN, NZ>), dim3((unsigned)blocks), dim3(256), lds, s, j0, j1,
+    hipLaunchKernelGGL((rfft2d_kernel<N, WIN, NZ, RAW>), dim3((unsigned)blocks), dim3(256), lds, s, j0, j1,
                        (unsigned)blocks0);
     return hipGetLastError();
+}
+
+template <int N, bool WIN, int NZ = N>
+static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
+{
+    if constexpr (!WIN && N <= 64) {
+        if (raw_ok(a) && (second == nullptr || raw_ok(*second))) return launch_fwd_impl<N, WIN, NZ, true>(a, second, s);
+    }
+    return launch_fwd_impl<N, WIN, NZ, false>(a, second, s);
 }
 
 template <int N, bool WIN>
