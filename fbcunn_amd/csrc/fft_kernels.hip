@@ -172,7 +172,8 @@ __device__ __forceinline__ void store_freq(float2 *p, const float2 &v)
 // lies, by LDS-direct loads (global_load_lds): no staging registers, no LDS store instructions and no
 // index arithmetic; the row pass then reads its rows at their (unaligned) places and masks the padding.
 // 16-byte pieces where the chunk allows (aligned16), 4-byte pieces for the rest.  The destination of a
-// wave instruction is wave-uniform; lane l lands at + l * size.
+// wave instruction is wave-uniform; lane l lands at + l * size.  AUX: cache policy bits (2 = non-temporal).
+template <int AUX>
 __device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloats, bool aligned16, int tid)
 {
     const int wave = tid >> 6, lane = tid & 63;
@@ -183,14 +184,14 @@ __device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloat
             if (p0 + lane < n16)
                 __builtin_amdgcn_global_load_lds(
                     (const void __attribute__((address_space(1))) *)(g + 4 * (p0 + lane)),
-                    (void __attribute__((address_space(3))) *)(raw + 4 * p0), 16, 0, 0);
+                    (void __attribute__((address_space(3))) *)(raw + 4 * p0), 16, 0, AUX);
         }
         done = n16 << 2;
     }
     for (int e0 = done + wave * 64; e0 < nfloats; e0 += 256) {
         if (e0 + lane < nfloats)
             __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(g + e0 + lane),
-                                             (void __attribute__((address_space(3))) *)(raw + e0), 4, 0, 0);
+                                             (void __attribute__((address_space(3))) *)(raw + e0), 4, 0, AUX);
     }
 }
 
@@ -354,7 +355,9 @@ __global__ __launch_bounds__(256, FftShape<N>::MIN_WAVES) void rfft2d_kernel(Fwd
         if constexpr (RAW) {
             // N floats of slack in front: the first row is read from -padL on
             float *raw = smem + N;
-            stage_raw(raw, in + (x0 + hs * S::TP) * hw, nph * hw, vec4 != 0, tid);
+            // N >= 64: planes of this size add up to tensors no cache holds until their next use, so
+            // they are streamed (non-temporal hint)
+            stage_raw<(N >= 64) ? 2 : 0>(raw, in + (x0 + hs * S::TP) * hw, nph * hw, vec4 != 0, tid);
             __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's pieces have landed
             __syncthreads();
             if (row_active && (t / S::TP) == hs) {
