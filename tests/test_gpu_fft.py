@@ -200,3 +200,19 @@ def test_1d_errors(nn):
     with pytest.raises(FbfcError) as e:
         nn.FFTWrapper("fbfft", 5, 0).fft(torch.zeros(3, 6, device="cuda"), torch.zeros(3, 5, 2, device="cuda"))
     assert e.value.code == ERR_INVALID_ARGUMENT
+
+
+def test_plane_count_beyond_the_32_bit_row_offsets_is_refused(nn):
+    """The kernels address one frequency row with 32-bit offsets: a plane count whose row would pass
+    2 GiB is refused before anything is launched (no buffer of that size is touched)."""
+    from fbcunn_amd._lib import FbfcError, lib
+    import ctypes
+    small = torch.zeros(1024, device="cuda")
+    planes = (1 << 31) // (5 * 8) + 1          # N = 8: (N/2+1) * planes * 8 bytes >= 2^31
+    rc = lib().fbfc_fft2d(ctypes.c_void_p(small.data_ptr()), planes, 1, 1, 0, 0, 8,
+                          ctypes.c_void_p(small.data_ptr()), ctypes.c_void_p(0))
+    assert rc != 0 and b"invalid" in lib().fbfc_last_error().lower()
+    rc = lib().fbfc_ifft2d(ctypes.c_void_p(small.data_ptr()), planes, 1, 1, 0, 0, 8,
+                           ctypes.c_void_p(small.data_ptr()), ctypes.c_void_p(0), 1, ctypes.c_void_p(0))
+    assert rc != 0
+    torch.cuda.synchronize()
