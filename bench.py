@@ -300,6 +300,29 @@ def measure_backward_step(nn, torch, synth, steps, warmup):
             "effective_tflops": 3 * 2.0 * B * F * P * o * o * k * k / (ms * 1e-3) / 1e12}
 
 
+def measure_reference_list(nn, torch, synth, steps):
+    """The layers of the reference's own benchmark list for this path (OverFeat-like, test/test_FFT.lua:440-448;
+    batch 128, memoryReuseNone): ms per pass and effective TFLOP/s of the three-pass step."""
+    layers = [(128, 96, 256, 5, 24, 2), (128, 256, 512, 3, 12, 1), (128, 512, 1024, 3, 12, 1), (128, 1024, 1024, 3, 12, 1)]
+    out = {}
+    for B, P, F, k, H, pad in layers:
+        o = H + 2 * pad - k + 1
+        net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad)
+        net.bias.zero_()
+        x = torch.from_numpy(synth.uniform(7, (B, P, H, H), stream=0)).cuda()
+        g = torch.from_numpy(synth.uniform(7, (B, F, o, o), stream=3)).cuda()
+        passes = ("fprop", "bprop", "accgrad")
+        n = max(3, steps // 5)
+        ms = time_loop(torch, lambda: [run_pass(net, x, g, p) for p in passes], n, 2)
+        per = {p: time_loop(torch, lambda: run_pass(net, x, g, p), n, 1) for p in passes}
+        flop = 2.0 * B * F * P * o * o * k * k
+        out["b%d_%dto%d_%dx%d_k%d_p%d" % (B, P, F, H, H, k, pad)] = {
+            "ms_per_step": ms, "ms_per_pass": per, "effective_tflops": 3 * flop / (ms * 1e-3) / 1e12,
+            "fft_size": net._plan_for(B, H, H).info.fft_size}
+        net.cleanupBuffers()
+    return out
+
+
 def measure_copy_bandwidth(torch):
     """A plain 256 MiB device-to-device copy: what HBM delivers to a trivial kernel on this box."""
     a = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
@@ -418,6 +441,7 @@ def main():
                 others[name] = measure_config(nn, torch, synth, name, max(5, args.steps // 5), 2)
         others["config2_fft_round_trip_8192x32x32"] = measure_fft_round_trip(nn, torch, synth, args.steps, args.warmup)
         others["tiled_convolution"] = measure_tiled(nn, torch, synth, args.steps, args.warmup)
+        others["reference_benchmark_layers"] = measure_reference_list(nn, torch, synth, args.steps)
         line["other_configs"] = others
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)
     print(json.dumps(line))
