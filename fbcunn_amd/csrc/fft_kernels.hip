@@ -48,10 +48,16 @@ struct FftShape {
     static constexpr int TP = T / PH;       // planes per staging round
     // waves per SIMD the register budget is sized for (N = 128 keeps 256 values per lane)
     static constexpr int MIN_WAVES = SMALL ? 2 : (N >= 128) ? 1 : (N == 32 && !INVERSE) ? 3 : PH;
-    // padding (in complex elements) between tile rows: keeps the T-lane groups
-    // of one wave on different LDS banks when T*8 bytes is below 128
-    static constexpr int ROWPAD = (T * 8 < 128) ? (64 / 8) / 2 : 0;
+    // padding (in complex elements) between tile rows.  Inverse: keeps the T-lane groups of one wave
+    // on different LDS banks when T*8 bytes is below 128.  Forward: a wave of the row pass holds TP
+    // planes (2 TP dwords side by side) of 64 / TP row pairs, two tile rows apart; a row stride of
+    // TP / 2 (mod 16) complex elements puts consecutive row pairs 2 TP banks apart, so the wave's
+    // 128 dwords tile the 64 banks exactly twice.
+    static constexpr int ROWPAD =
+        INVERSE ? ((T * 8 < 128) ? (64 / 8) / 2 : 0) : (TP >= 32) ? 0 : (TP >= 2) ? TP / 2 : 1;
     static constexpr int ROWSTRIDE = KXP * T + ROWPAD;  // complex elements
+    // lanes of one staging round (the row pass of round r runs on waves [r LPR/64, (r+1) LPR/64))
+    static constexpr int LPR = THREADS / PH;
 };
 
 // LDS staging area in canvas-row layout.  Row (p*h + r) of the staged planes starts at
@@ -327,14 +333,14 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
     if constexpr (WIN) {
         if (win.on) build_window_table<N>(tbl, win, x0, planes, tid);
     }
-    const int y_lo = padU & ~1;                       // first canvas row that can be non-zero (even)
-    const int y_hi = (padU + h + 1) & ~1;             // one past the last, rounded up to even
-
-    const int t = tid % T;
     float re[N], im[N];
 
-    // ---- row pass: lane (t, rp) owns canvas rows 2rp and 2rp+1 of plane t ----
-    const int rp = tid / T;
+    // ---- row pass: lane (t, rp) owns canvas rows 2rp and 2rp+1 of plane t.  The planes are staged
+    // TP at a time; the lanes of round r are LPR consecutive ones (whole waves), so a wave runs the
+    // row reads of its own round only ----
+    const int round_of_lane = tid / S::LPR, rl = tid % S::LPR;
+    const int t = round_of_lane * S::TP + rl % S::TP;
+    const int rp = rl / S::TP;
     const int ya = 2 * rp, yb = ya + 1;
     const int ia = ya - padU, ib = yb - padU;
     const bool va = (ia >= 0) && (ia < h);
@@ -349,30 +355,35 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
     // as zero-padded canvas rows.
     static_assert(!RAW || (!WIN && N <= 64), "raw staging: plain operands, N <= 64");
     const int zrow = S::TP * h;  // canvas staging: an all-zero row for canvas rows outside the plane
+    // raw staging: bit x of colmask = canvas column x lies inside the plane
+    [[maybe_unused]] const unsigned long long colmask = ((w >= 64) ? ~0ull : ((1ull << w) - 1ull)) << padL;
     static_for<S::PH>([&](auto hh) {
         constexpr int hs = decltype(hh)::value;
         int nph = np - hs * S::TP;
         nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
         if (hs > 0) __syncthreads();  // previous round fully read
         if constexpr (RAW) {
-            // N floats of slack in front: the first row is read from -padL on
+            // N floats of slack on either side of the chunk (the first row is read from -padL on, the last
+            // one up to N - 1 - padL), then N zeros for the canvas rows outside the plane
             float *raw = smem + N;
+            float *zeros = raw + S::TP * hw + N;
+            if (hs == 0 && tid < N) zeros[tid] = 0.0f;
             // N >= 64: planes of this size add up to tensors no cache holds until their next use, so
             // they are streamed (non-temporal hint)
             stage_raw<(N >= 64) ? 2 : 0>(raw, in + (x0 + hs * S::TP) * hw, nph * hw, vec4 != 0, tid);
             __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's pieces have landed
             __syncthreads();
-            if (row_active && (t / S::TP) == hs) {
+            if (row_active && round_of_lane == hs) {
                 const int tl = t - hs * S::TP;
-                const float *pa = raw + (va ? (tl * h + ia) * w : 0) - padL;
-                const float *pb = raw + (vb ? (tl * h + ib) * w : 0) - padL;
+                const float *pa = va ? raw + (tl * h + ia) * w - padL : zeros;
+                const float *pb = vb ? raw + (tl * h + ib) * w - padL : zeros;
                 static_for<N>([&](auto xx) {
                     constexpr int x = decltype(xx)::value;
                     if constexpr (x < NZ) {
-                        const float a = pa[x], b = pb[x];
-                        const bool cx = (unsigned)(x - padL) < (unsigned)w;  // column inside the plane
-                        re[x] = (va && cx) ? a : 0.0f;
-                        im[x] = (vb && cx) ? b : 0.0f;
+                        // what lies left and right of the row in LDS is masked off bit-wise
+                        const unsigned m = ((colmask >> x) & 1ull) ? 0xffffffffu : 0u;
+                        re[x] = __uint_as_float(__float_as_uint(pa[x]) & m);
+                        im[x] = __uint_as_float(__float_as_uint(pb[x]) & m);
                     } else {
                         re[x] = 0.0f;
                         im[x] = 0.0f;
@@ -391,7 +402,7 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
                 copy_canvas<N, true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
             }
             __syncthreads();
-            if (row_active && (t / S::TP) == hs) {
+            if (row_active && round_of_lane == hs) {
                 const int tl = t - hs * S::TP;
                 const float4 *pa = reinterpret_cast<const float4 *>(smem + (va ? tl * h + ia : zrow) * LDR);
                 const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? tl * h + ib : zrow) * LDR);
@@ -413,16 +424,17 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
     // ---- row FFT and untangling ----
     // A[k] / B[k]: spectra of rows ya / yb; slot 0 carries the real-valued columns 0 and N/2.
     // The first phase's columns go straight to the LDS tile, later ones wait in registers.
+    // The tile R[y][kx][t] holds every canvas row the column pass reads (all N, or NZ for small
+    // planes) at a fixed place, so the column pass addresses it with compile-time offsets; the lanes
+    // whose two rows lie outside the plane write the zeros.
     constexpr int NLATE = S::NH2 - S::KXP;  // 0 when there is a single phase
+    constexpr int TROWS = (NZ < N) ? NZ : N;
     float ar[NLATE > 0 ? NLATE : 1], ai[NLATE > 0 ? NLATE : 1], br[NLATE > 0 ? NLATE : 1], bi[NLATE > 0 ? NLATE : 1];
     float2 *R = reinterpret_cast<float2 *>(smem);
-    const int kx = tid / T;  // column pass: lane (t, kx) owns tile column kx of plane t
-    const int nrows = y_hi - y_lo;  // tile rows; row index nrows is an all-zero row
     __syncthreads();  // staging area fully consumed; the tile may overwrite it
-    if (tid < S::KXP * T) R[nrows * S::ROWSTRIDE + tid] = make_float2(0.0f, 0.0f);
     if (row_active) {
         fft_inplace_nz<N, NZ, false>(re, im);
-        float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
+        float2 *Ra = R + ya * S::ROWSTRIDE + t;
         float2 *Rb = Ra + S::ROWSTRIDE;
         Ra[0] = make_float2(re[brev<N>(0)], re[brev<N>(N / 2)]);
         Rb[0] = make_float2(im[brev<N>(0)], im[brev<N>(N / 2)]);
@@ -439,16 +451,28 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
                 br[k - S::KXP] = 0.5f * (zi + ni);  bi[k - S::KXP] = 0.5f * (nr - zr);
             }
         });
+    } else if (t < np && ya < TROWS) {
+        // both rows are zero in every phase: written once, the refills below leave them alone
+        float2 *Ra = R + ya * S::ROWSTRIDE + t;
+        float2 *Rb = Ra + S::ROWSTRIDE;
+        static_for<S::KXP>([&](auto kk) {
+            constexpr int k = decltype(kk)::value;
+            Ra[k * T] = make_float2(0.0f, 0.0f);
+            Rb[k * T] = make_float2(0.0f, 0.0f);
+        });
     }
 
     // Each phase: (later phases first refill the tile from registers) then the lanes whose
     // column belongs to the phase pull it into registers, which frees the tile again.
+    // Column pass: lane (tc, kx) owns tile column kx of plane tc.
+    const int tc = tid % T;
+    const int kx = tid / T;
     static_for<S::PH>([&](auto pp) {
         constexpr int ph = decltype(pp)::value;
         if constexpr (ph > 0) {
             __syncthreads();  // previous phase's columns are in registers
             if (row_active) {
-                float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
+                float2 *Ra = R + ya * S::ROWSTRIDE + t;
                 float2 *Rb = Ra + S::ROWSTRIDE;
                 static_for<S::KXP>([&](auto kk) {
                     constexpr int kl = decltype(kk)::value;
@@ -459,15 +483,13 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
             }
         }
         __syncthreads();
-        if ((t < np) && (kx / S::KXP) == ph) {
+        if ((tc < np) && (kx / S::KXP) == ph) {
             const int kl = kx - ph * S::KXP;
-            const float2 *col = R + kl * T + t;
+            const float2 *col = R + kl * T + tc;
             static_for<N>([&](auto yy) {
                 constexpr int y = decltype(yy)::value;
                 if constexpr (y < NZ) {
-                    // canvas rows outside the plane read the zero row (uniform select, no branch)
-                    const int row = ((y >= y_lo) && (y < y_hi)) ? (y - y_lo) : nrows;
-                    const float2 v = col[row * S::ROWSTRIDE];
+                    const float2 v = col[y * S::ROWSTRIDE];
                     re[y] = v.x;
                     im[y] = v.y;
                 } else {
@@ -479,11 +501,11 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
     });
 
     // ---- column FFT and frequency-major store, all lanes at once ----
-    if (t < np) {
+    if (tc < np) {
         fft_inplace_nz<N, NZ, false>(re, im);
         // address = uniform base (frequency row ky, first plane of the group) + 32-bit lane offset
-        const unsigned voff = (unsigned)(((long)kx * planes + t) * (long)sizeof(float2));
-        const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + t) * (long)sizeof(float2));
+        const unsigned voff = (unsigned)(((long)kx * planes + tc) * (long)sizeof(float2));
+        const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + tc) * (long)sizeof(float2));
         char *obase = reinterpret_cast<char *>(out + x0);
         const long rowbytes = (long)S::NH * planes * (long)sizeof(float2);
         if (kx != 0) {
@@ -675,11 +697,12 @@ static size_t fft_lds_bytes(int h, int w, int padU)
 {
     using S = FftShape<N, INVERSE, SMALL>;
     const int y_lo = padU & ~1, y_hi = (padU + h + 1) & ~1;
-    const size_t tile = (size_t)(y_hi - y_lo + 1) * S::ROWSTRIDE * sizeof(float2);
+    // inverse: the canvas rows of the plane and a zero row; forward: every row the column pass reads
+    const size_t tile = (INVERSE ? (size_t)(y_hi - y_lo + 1) : (size_t)(SMALL ? 16 : N)) * S::ROWSTRIDE * sizeof(float2);
     // canvas-row staging (the inverse, windowed operands, N = 128) or, smaller, the raw chunk with N
-    // floats of slack on either side
+    // floats of slack on either side and N zeros behind
     const size_t canvas = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
-    const size_t raw = ((size_t)S::TP * h * w + 2 * N) * sizeof(float);
+    const size_t raw = ((size_t)S::TP * h * w + 3 * N) * sizeof(float);
     const size_t stage = canvas > raw ? canvas : raw;
     return ((tile > stage ? tile : stage) + 15) & ~(size_t)15;
 }
