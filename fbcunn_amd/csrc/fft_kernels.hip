@@ -34,8 +34,13 @@ namespace fbfc {
 // all columns fit at once, so it runs in one phase (144 -> 137 us for 24576 planes of 9 x 9).
 template <int N, bool INVERSE = false, bool SMALL = false>
 struct FftShape {
-    static constexpr int T = 512 / N;       // planes per workgroup
-    static constexpr int THREADS = 256;     // T * N / 2
+    // planes per workgroup: 256 lanes' worth, except N = 64, which takes 16 planes (512 lanes) so
+    // that its runs per frequency are whole 128-byte lines -- measured with the bare
+    // access pattern (contiguous reads, frequency-major writes, no arithmetic) at 16384 planes of
+    // 47 x 47: 123 us with 64-byte runs from two 256-lane workgroups per CU, 89 us with 128-byte runs
+    // from one 512-lane workgroup; at 24576 planes of 9 x 9: 128 against 90 us
+    static constexpr int T = (N == 64) ? 16 : 512 / N;
+    static constexpr int THREADS = T * N / 2;
     static constexpr int NH2 = N / 2;       // complex slots per tile row
     static constexpr int NH = N / 2 + 1;    // stored column frequencies
     // (N = 32 forward: two phases halve the LDS footprint and a third workgroup fits a CU, measured
@@ -48,13 +53,11 @@ struct FftShape {
     static constexpr int TP = T / PH;       // planes per staging round
     // waves per SIMD the register budget is sized for (N = 128 keeps 256 values per lane)
     static constexpr int MIN_WAVES = SMALL ? 2 : (N >= 128) ? 1 : (N == 32 && !INVERSE) ? 3 : PH;
-    // padding (in complex elements) between tile rows.  Inverse: keeps the T-lane groups of one wave
-    // on different LDS banks when T*8 bytes is below 128.  Forward: a wave of the row pass holds TP
-    // planes (2 TP dwords side by side) of 64 / TP row pairs, two tile rows apart; a row stride of
+    // padding (in complex elements) between tile rows.  A wave of the row pass holds TP planes
+    // (2 TP dwords side by side) of 64 / TP row pairs, two tile rows apart; a row stride of
     // TP / 2 (mod 16) complex elements puts consecutive row pairs 2 TP banks apart, so the wave's
     // 128 dwords tile the 64 banks exactly twice.
-    static constexpr int ROWPAD =
-        INVERSE ? ((T * 8 < 128) ? (64 / 8) / 2 : 0) : (TP >= 32) ? 0 : (TP >= 2) ? TP / 2 : 1;
+    static constexpr int ROWPAD = (TP >= 32) ? 0 : (TP >= 2) ? TP / 2 : 1;
     static constexpr int ROWSTRIDE = KXP * T + ROWPAD;  // complex elements
     // lanes of one staging round (the row pass of round r runs on waves [r LPR/64, (r+1) LPR/64))
     static constexpr int LPR = THREADS / PH;
@@ -74,10 +77,10 @@ struct Canvas {
 // group's run per frequency is only half a 128-byte line (T*8 = 64 bytes), the two groups that
 // share each line are given to workgroups b and b+8: same XCD, dispatched back to back, so the
 // two halves meet in that XCD's L2 (one line fetched once / written back whole).
-template <int N>
+template <int T>
 __device__ __forceinline__ long plane_group(unsigned bid)
 {
-    if constexpr (FftShape<N>::T * 8 >= 128) {
+    if constexpr (T * 8 >= 128) {
         return (long)bid;
     } else {
         const unsigned cyc = bid >> 4, r = bid & 15u;
@@ -85,7 +88,7 @@ __device__ __forceinline__ long plane_group(unsigned bid)
     }
 }
 
-template <int N, bool TO_LDS>
+template <int N, bool TO_LDS, int NT = 256>
 __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, int w, int padL,
                                             int vec4, int tid)
 {
@@ -96,16 +99,16 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
         const int n4 = total >> 2;
         float4 *g4 = reinterpret_cast<float4 *>(g);
         int row = (tid * 4) / w, x = tid * 4 - row * w;
-        const int drow = 1024 / w, dx = 1024 - drow * w;
+        const int drow = (4 * NT) / w, dx = 4 * NT - drow * w;
         if constexpr (TO_LDS) {
             // U loads in flight per lane before the first one is waited for: one load per round trip
             // would leave the memory system idle for most of the copy
             constexpr int U = (N >= 64) ? 12 : 8;
-            for (int i0 = tid; i0 < n4; i0 += 256 * U) {
+            for (int i0 = tid; i0 < n4; i0 += NT * U) {
                 float4 q[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    const int i = i0 + 256 * u;
+                    const int i = i0 + NT * u;
                     if (i < n4) {
                         if constexpr (N >= 64) {
                             // planes of this size add up to tensors no cache holds until their next use:
@@ -120,7 +123,7 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    const int i = i0 + 256 * u;
+                    const int i = i0 + NT * u;
                     if (i < n4) {
                         const float v[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
                         int r_ = row, x_ = x;
@@ -136,7 +139,7 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
                 }
             }
         } else {
-            for (int i = tid; i < n4; i += 256) {
+            for (int i = tid; i < n4; i += NT) {
                 float v[4];
                 int r_ = row, x_ = x;
 #pragma unroll
@@ -155,8 +158,8 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
     {
         const int first = done + tid;
         int row = first / w, x = first - row * w;
-        const int drow = 256 / w, dx = 256 - drow * w;
-        for (int i = first; i < total; i += 256) {
+        const int drow = NT / w, dx = NT - drow * w;
+        for (int i = first; i < total; i += NT) {
             float *sp = smem + row * LDR + padL + x;
             if (TO_LDS) *sp = g[i]; else g[i] = *sp;
             row += drow;
@@ -172,7 +175,7 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
 template <int N>
 __device__ __forceinline__ void store_freq(float2 *p, const float2 &v)
 {
-    if constexpr (FftShape<N>::T * 8 >= 128) store_nt(p, v);
+    if constexpr (FftShape<N, false>::T * 8 >= 128) store_nt(p, v);
     else *p = v;
 }
 
@@ -181,14 +184,14 @@ __device__ __forceinline__ void store_freq(float2 *p, const float2 &v)
 // index arithmetic; the row pass then reads its rows at their (unaligned) places and masks the padding.
 // 16-byte pieces where the chunk allows (aligned16), 4-byte pieces for the rest.  The destination of a
 // wave instruction is wave-uniform; lane l lands at + l * size.  AUX: cache policy bits (2 = non-temporal).
-template <int AUX>
+template <int AUX, int NT = 256>
 __device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloats, bool aligned16, int tid)
 {
     const int wave = tid >> 6, lane = tid & 63;
     int done = 0;
     if (aligned16) {
         const int n16 = nfloats >> 2;
-        for (int p0 = wave * 64; p0 < n16; p0 += 256) {
+        for (int p0 = wave * 64; p0 < n16; p0 += NT) {
             if (p0 + lane < n16)
                 __builtin_amdgcn_global_load_lds(
                     (const void __attribute__((address_space(1))) *)(g + 4 * (p0 + lane)),
@@ -196,7 +199,7 @@ __device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloat
         }
         done = n16 << 2;
     }
-    for (int e0 = done + wave * 64; e0 < nfloats; e0 += 256) {
+    for (int e0 = done + wave * 64; e0 < nfloats; e0 += NT) {
         if (e0 + lane < nfloats)
             __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(g + e0 + lane),
                                              (void __attribute__((address_space(3))) *)(raw + e0), 4, 0, AUX);
@@ -204,12 +207,12 @@ __device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloat
 }
 
 // Zeroes the margins of nrows canvas rows and the all-zero row kept at index zrow.
-template <int N>
+template <int N, int NT = 256>
 __device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int w, int padL, int zrow,
                                                     int tid)
 {
     constexpr int LDR = Canvas<N>::LDR;
-    for (int row = tid; row < nrows; row += 256) {
+    for (int row = tid; row < nrows; row += NT) {
         float *sp = smem + row * LDR;
         for (int c = 0; c < padL; ++c) sp[c] = 0.0f;
         for (int c = padL + w; c < N; ++c) sp[c] = 0.0f;
@@ -309,14 +312,15 @@ struct FwdJob {
 // NZ < N: planes of at most NZ x NZ at the canvas origin (convolution kernels): the transforms skip
 // the inputs that are known to be zero.
 template <int N, bool WIN, int NZ, bool RAW>
-__global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) void rfft2d_kernel(FwdJob job0, FwdJob job1,
+__global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<N, false, (NZ < N)>::MIN_WAVES)) void rfft2d_kernel(FwdJob job0, FwdJob job1,
                                                                       unsigned blocks0)
 {
     using S = FftShape<N, false, (NZ < N)>;
     constexpr int T = S::T;
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x;
-    const bool second = blockIdx.x >= blocks0;
+    const unsigned v = blockIdx.x;
+    const bool second = v >= blocks0;
     const float *__restrict__ in = second ? job1.in : job0.in;
     float2 *__restrict__ out = second ? job1.out : job0.out;
     const long planes = second ? job1.planes : job0.planes;
@@ -324,7 +328,7 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
     const int padU = second ? job1.padU : job0.padU, padL = second ? job1.padL : job0.padL;
     const int vec4 = second ? job1.vec4 : job0.vec4;
     const int herm = second ? job1.herm : job0.herm;
-    const long x0 = plane_group<N>(blockIdx.x - (second ? blocks0 : 0u)) * T;
+    const long x0 = plane_group<T>(v - (second ? blocks0 : 0u)) * T;
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
@@ -370,7 +374,7 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
             if (hs == 0 && tid < N) zeros[tid] = 0.0f;
             // N >= 64: planes of this size add up to tensors no cache holds until their next use, so
             // they are streamed (non-temporal hint)
-            stage_raw<(N >= 64) ? 2 : 0>(raw, in + (x0 + hs * S::TP) * hw, nph * hw, vec4 != 0, tid);
+            stage_raw<(N >= 64) ? 2 : 0, S::THREADS>(raw, in + (x0 + hs * S::TP) * hw, nph * hw, vec4 != 0, tid);
             __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's pieces have landed
             __syncthreads();
             if (row_active && round_of_lane == hs) {
@@ -395,11 +399,11 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
             if constexpr (WIN) windowed = win.on != 0;
             if (windowed) {
                 if (hs == 0) __syncthreads();  // window table complete
-                zero_canvas_margins<N>(smem, 0, w, 0, zrow, tid);  // the all-zero row only
+                zero_canvas_margins<N, S::THREADS>(smem, 0, w, 0, zrow, tid);  // the all-zero row only
                 copy_windows<N, true>(smem, const_cast<float *>(in), tbl, hs * S::TP, nph, h, w, 0, win, tid);
             } else {
-                zero_canvas_margins<N>(smem, nph * h, w, padL, zrow, tid);
-                copy_canvas<N, true>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
+                zero_canvas_margins<N, S::THREADS>(smem, nph * h, w, padL, zrow, tid);
+                copy_canvas<N, true, S::THREADS>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
             }
             __syncthreads();
             if (row_active && round_of_lane == hs) {
@@ -538,7 +542,7 @@ __global__ __launch_bounds__(256, (FftShape<N, false, (NZ < N)>::MIN_WAVES)) voi
 // real[r][s] = y[r+padU][s+padL] (+ bias[plane % bias_period])
 // ---------------------------------------------------------------------------------
 template <int N, bool WIN>
-__global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_kernel(const float2 *__restrict__ in,
+__global__ __launch_bounds__((FftShape<N, true>::THREADS), (FftShape<N, true>::MIN_WAVES)) void irfft2d_kernel(const float2 *__restrict__ in,
                                                       float *__restrict__ out, long planes,
                                                       int h, int w, int padU, int padL,
                                                       const float *__restrict__ bias,
@@ -555,7 +559,7 @@ __global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_k
         return;
     }
     const int tid = threadIdx.x;
-    const long x0 = plane_group<N>(blockIdx.x - bgrad_blocks) * T;
+    const long x0 = plane_group<T>(blockIdx.x - bgrad_blocks) * T;
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
@@ -564,9 +568,6 @@ __global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_k
         // read again only after the barriers of the passes below
         if (win.on) build_window_table<N>(tbl, win, x0, planes, tid);
     }
-    const int y_lo = padU & ~1;                       // canvas rows the crop needs
-    const int y_hi = (padU + h + 1) & ~1;
-
     const int t = tid % T;
     float re[N], im[N];
     float2 *R = reinterpret_cast<float2 *>(smem);
@@ -604,16 +605,19 @@ __global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_k
         fft_inplace<N, true>(re, im);
     }
 
-    // ---- row pass bookkeeping: lane (t, rp) rebuilds canvas rows 2rp, 2rp+1 ----
-    const int rp = tid / T;
+    // ---- row pass bookkeeping: lane (tr, rp) rebuilds canvas rows 2rp, 2rp+1 of plane tr.  The
+    // planes leave TP at a time; the lanes of round r are LPR consecutive ones (whole waves), so a wave
+    // runs the staging writes of its own round only ----
+    const int round_of_lane = tid / S::LPR, rl = tid % S::LPR;
+    const int tr = round_of_lane * S::TP + rl % S::TP;
+    const int rp = rl / S::TP;
     const int ya = 2 * rp, yb = ya + 1;
     const int ia = ya - padU, ib = yb - padU;
     const bool va = (ia >= 0) && (ia < h);
     const bool vb = (ib >= 0) && (ib < h);
-    const bool row_active = (t < np) && (va || vb);
+    const bool row_active = (tr < np) && (va || vb);
     // Z[k] = Ya[k] + i Yb[k], k = 0..N-1, with Y[N-k] = conj Y[k]
     float zr[N], zi[N];
-    const int nrows = y_hi - y_lo;  // tile rows; row index nrows is a dummy row
 
     static_for<S::PH>([&](auto pp) {
         constexpr int ph = decltype(pp)::value;
@@ -621,16 +625,15 @@ __global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_k
         if ((t < np) && (kx / S::KXP) == ph) {
             const int kl = kx - ph * S::KXP;
             float2 *col = R + kl * T + t;
+            // every canvas row has its fixed place in the tile R[y][kx][t]: compile-time offsets
             static_for<N>([&](auto yy) {
                 constexpr int y = decltype(yy)::value;
-                // rows the crop does not need land in a dummy row (uniform select, no branch)
-                const int row = ((y >= y_lo) && (y < y_hi)) ? (y - y_lo) : nrows;
-                col[row * S::ROWSTRIDE] = make_float2(re[brev<N>(y)], im[brev<N>(y)]);
+                col[y * S::ROWSTRIDE] = make_float2(re[brev<N>(y)], im[brev<N>(y)]);
             });
         }
         __syncthreads();
         if (row_active) {
-            const float2 *Ra = R + (ya - y_lo) * S::ROWSTRIDE + t;
+            const float2 *Ra = R + ya * S::ROWSTRIDE + tr;
             const float2 *Rb = Ra + S::ROWSTRIDE;
             static_for<S::KXP>([&](auto kk) {
                 constexpr int kl = decltype(kk)::value;
@@ -651,7 +654,7 @@ __global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_k
     float bv = 0.0f;
     if (row_active) {
         fft_inplace<N, true>(zr, zi);
-        if (bias != nullptr) bv = bias[(x0 + t) % bias_period];
+        if (bias != nullptr) bv = bias[(x0 + tr) % bias_period];
     }
     // ---- canvas rows (+bias) into the staging area, cropped coalesced copy-out, TP planes per round ----
     constexpr int LDR = Canvas<N>::LDR;
@@ -660,8 +663,8 @@ __global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_k
         int nph = np - hs * S::TP;
         nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
         if (hs > 0) __syncthreads();  // previous round copied out
-        if (row_active && (t / S::TP) == hs) {
-            const int tl = t - hs * S::TP;
+        if (row_active && round_of_lane == hs) {
+            const int tl = tr - hs * S::TP;
             if (va) {
                 float4 *pa = reinterpret_cast<float4 *>(smem + (tl * h + ia) * LDR);
                 static_for<N / 4>([&](auto jj) {
@@ -685,7 +688,7 @@ __global__ __launch_bounds__(256, (FftShape<N, true>::MIN_WAVES)) void irfft2d_k
         if (windowed)
             copy_windows<N, false>(smem, out, tbl, hs * S::TP, nph, h, w, padL, win, tid);
         else
-            copy_canvas<N, false>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
+            copy_canvas<N, false, S::THREADS>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
     });
 }
 
@@ -696,9 +699,9 @@ template <int N, bool INVERSE, bool SMALL = false>
 static size_t fft_lds_bytes(int h, int w, int padU)
 {
     using S = FftShape<N, INVERSE, SMALL>;
-    const int y_lo = padU & ~1, y_hi = (padU + h + 1) & ~1;
-    // inverse: the canvas rows of the plane and a zero row; forward: every row the column pass reads
-    const size_t tile = (INVERSE ? (size_t)(y_hi - y_lo + 1) : (size_t)(SMALL ? 16 : N)) * S::ROWSTRIDE * sizeof(float2);
+    (void)padU;
+    // the tile holds every canvas row at a fixed place (the rows the small-plane forward variant reads)
+    const size_t tile = (size_t)(SMALL ? 16 : N) * S::ROWSTRIDE * sizeof(float2);
     // canvas-row staging (the inverse, windowed operands, N = 128) or, smaller, the raw chunk with N
     // floats of slack on either side and N zeros behind
     const size_t canvas = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
@@ -710,7 +713,7 @@ static size_t fft_lds_bytes(int h, int w, int padU)
 template <int N>
 static long fwd_blocks(long planes)
 {
-    using S = FftShape<N>;
+    using S = FftShape<N, false>;
     long blocks = (planes + S::T - 1) / S::T;
     if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
     return blocks;
@@ -719,7 +722,7 @@ static long fwd_blocks(long planes)
 template <int N>
 static FwdJob make_job(const FwdArgs &a)
 {
-    using S = FftShape<N>;
+    using S = FftShape<N, false>;
     FwdJob j;
     j.in = a.in;
     j.out = reinterpret_cast<float2 *>(a.out);
@@ -769,7 +772,7 @@ static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipSt
         lds += FftShape<N>::T * sizeof(int4);
     }
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((rfft2d_kernel<N, WIN, NZ, RAW>), dim3((unsigned)blocks), dim3(256), lds, s, j0, j1,
+    hipLaunchKernelGGL((rfft2d_kernel<N, WIN, NZ, RAW>), dim3((unsigned)blocks), dim3(FftShape<N, false, (NZ < N)>::THREADS), lds, s, j0, j1,
                        (unsigned)blocks0);
     return hipGetLastError();
 }
@@ -804,7 +807,7 @@ static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
                                a.out_planes};
     const unsigned bblocks = (bgrad.dc != nullptr) ? bias_grad_dc_blocks(bgrad.planes) : 0u;
     if (blocks + bblocks > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((irfft2d_kernel<N, WIN>), dim3((unsigned)blocks + bblocks), dim3(256), lds, s,
+    hipLaunchKernelGGL((irfft2d_kernel<N, WIN>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
                        reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL,
                        a.bias, a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks, a.win, tbl_off);
     return hipGetLastError();
