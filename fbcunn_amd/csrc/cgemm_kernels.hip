@@ -213,6 +213,39 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
 }
 
 // ---------------------------------------------------------------------------------------
+// Complex products with three real MFMAs instead of four.  With
+//   P1 = sum ar br,  P2 = sum ai bi,  P3 = sum (ar +- ai)(br +- bi)
+// the three modes are
+//   A conj(B):     Re = P1 + P2,  Im = P3 - P1 + P2,  P3 from (ar + ai)(br - bi)
+//   A B:           Re = P1 - P2,  Im = P3 - P1 - P2,  P3 from (ar + ai)(br + bi)
+//   conj(A)^T B:   Re = P1 + P2,  Im = P3 - P1 + P2,  P3 from (ar - ai)(br + bi)
+// i.e. 6 instead of 8 flops per complex multiply-add on the matrix cores, paid for with two
+// vector adds per operand element and a third accumulator (16 registers per 32x32 block).
+// ---------------------------------------------------------------------------------------
+template <int MODE>
+__device__ __forceinline__ void cmac3(float ar, float ai, float br, float bi, floatx16 &p1, floatx16 &p2,
+                                      floatx16 &p3)
+{
+    const float sa = (MODE == 2) ? ar - ai : ar + ai;
+    const float sb = (MODE == 0) ? br - bi : br + bi;
+    p1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, p1, 0, 0, 0);
+    p2 = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, bi, p2, 0, 0, 0);
+    p3 = __builtin_amdgcn_mfma_f32_32x32x2f32(sa, sb, p3, 0, 0, 0);
+}
+
+template <int MODE>
+__device__ __forceinline__ void combine3(const floatx16 &p1, const floatx16 &p2, const floatx16 &p3,
+                                         floatx16 &cre, floatx16 &cim)
+{
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const float s2 = (MODE == 1) ? -p2[r] : p2[r];
+        cre[r] = p1[r] + s2;
+        cim[r] = (p3[r] - p1[r]) + s2;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // LDS-direct variant of the tiled kernel (M % 64 == N % 64 == 0, K % 16 == 0).
 //
 // Operand tiles go from global memory straight into LDS with global_load_lds_dwordx4: no
@@ -286,9 +319,9 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
     const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, h = lane >> 5;
 
-    floatx16 cre, cim;
+    floatx16 p1, p2, p3;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { cre[r] = 0.f; cim[r] = 0.f; }
+    for (int r = 0; r < 16; ++r) { p1[r] = 0.f; p2[r] = 0.f; p3[r] = 0.f; }
 
     const int nk = K / KT;
     auto issue = [&](int kt, int buf) {
@@ -325,12 +358,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
                 b[4 * j] = vb.x; b[4 * j + 1] = vb.y; b[4 * j + 2] = vb.z; b[4 * j + 3] = vb.w;
             }
 #pragma unroll
-            for (int s = 0; s < 16; s += 2) {
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], -b[s + 1], cim, 0, 0, 0);
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s + 1], b[s + 1], cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s + 1], b[s], cim, 0, 0, 0);
-            }
+            for (int s = 0; s < 16; s += 2) cmac3<0>(a[s], a[s + 1], b[s], b[s + 1], p1, p2, p3);
         } else if (MODE == 1) {
             float a[16];
 #pragma unroll
@@ -341,10 +369,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) {
                 const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDB + 2 * bcol);
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.x, cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.y, cim, 0, 0, 0);
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], -vb.y, cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], vb.x, cim, 0, 0, 0);
+                cmac3<1>(a[2 * kk], a[2 * kk + 1], vb.x, vb.y, p1, p2, p3);
             }
         } else {
 #pragma unroll
@@ -352,10 +377,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
                 // half-wave h owns k = 8h + kk: both components of conj(A)[k][arow] and B[k][bcol]
                 const float2 va = *reinterpret_cast<const float2 *>(as + (8 * h + kk) * LDM + 2 * arow);
                 const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDB + 2 * bcol);
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(va.x, vb.x, cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(va.x, vb.y, cim, 0, 0, 0);
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(va.y, vb.y, cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(va.y, -vb.x, cim, 0, 0, 0);
+                cmac3<2>(va.x, va.y, vb.x, vb.y, p1, p2, p3);
             }
         }
         if (kt + 1 < nk) {
@@ -364,6 +386,8 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
         }
     }
 
+    floatx16 cre, cim;
+    combine3<MODE>(p1, p2, p3, cre, cim);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int row = m0 + 32 * wm + 8 * (r / 4) + 4 * h + (r % 4);
@@ -449,29 +473,11 @@ __device__ __forceinline__ void splitk_load(const float2 *__restrict__ Aq, const
 }
 
 template <int MODE>
-__device__ __forceinline__ void splitk_mfma(const float (&a)[16], const float (&b)[16], floatx16 &cre,
-                                            floatx16 &cim)
+__device__ __forceinline__ void splitk_mfma(const float (&a)[16], const float (&b)[16], floatx16 &p1,
+                                            floatx16 &p2, floatx16 &p3)
 {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const float ar = a[2 * j], ai = a[2 * j + 1], br = b[2 * j], bi = b[2 * j + 1];
-        if (MODE == 0) {         // A conj(B)
-            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, cre, 0, 0, 0);
-            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, -bi, cim, 0, 0, 0);
-            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, bi, cre, 0, 0, 0);
-            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, br, cim, 0, 0, 0);
-        } else if (MODE == 1) {  // A B
-            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, cre, 0, 0, 0);
-            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, bi, cim, 0, 0, 0);
-            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, -bi, cre, 0, 0, 0);
-            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, br, cim, 0, 0, 0);
-        } else {                 // conj(A)^T B
-            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, cre, 0, 0, 0);
-            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, bi, cim, 0, 0, 0);
-            cre = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, bi, cre, 0, 0, 0);
-            cim = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, -br, cim, 0, 0, 0);
-        }
-    }
+    for (int j = 0; j < 8; ++j) cmac3<MODE>(a[2 * j], a[2 * j + 1], b[2 * j], b[2 * j + 1], p1, p2, p3);
 }
 
 // red: [wave][accumulator register][lane] partial sums (used when SK > 1)
@@ -501,9 +507,9 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
     const int kq = K / SK;                    // this wave's share of K (a multiple of 16)
     const int kbeg = ks * kq, nkt = kq >> 4;  // K-tiles of 16 complex
 
-    floatx16 cre, cim;
+    floatx16 p1, p2, p3;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { cre[r] = 0.f; cim[r] = 0.f; }
+    for (int r = 0; r < 16; ++r) { p1[r] = 0.f; p2[r] = 0.f; p3[r] = 0.f; }
 
     if (live) {
         if constexpr (SK == 1) {
@@ -514,26 +520,29 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
             for (; kt + 1 < nkt; kt += 2) {
                 splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * (kt + 1), h, a1, b1);
                 __builtin_amdgcn_sched_barrier(0);
-                splitk_mfma<MODE>(a0, b0, cre, cim);
+                splitk_mfma<MODE>(a0, b0, p1, p2, p3);
                 __builtin_amdgcn_sched_barrier(0);
                 // the last prefetch of an even count re-reads the final tile and is not used
                 const int knext = (kt + 2 < nkt) ? kt + 2 : kt + 1;
                 splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * knext, h, a0, b0);
                 __builtin_amdgcn_sched_barrier(0);
-                splitk_mfma<MODE>(a1, b1, cre, cim);
+                splitk_mfma<MODE>(a1, b1, p1, p2, p3);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (kt < nkt) splitk_mfma<MODE>(a0, b0, cre, cim);
+            if (kt < nkt) splitk_mfma<MODE>(a0, b0, p1, p2, p3);
         } else {
             // one to four K-tiles per wave: the compiler interleaves each tile's loads with the
             // previous tile's MFMAs, and at about 64 registers per lane five workgroups share a CU
             float a[16], b[16];
             for (int kt = 0; kt < nkt; ++kt) {
                 splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * kt, h, a, b);
-                splitk_mfma<MODE>(a, b, cre, cim);
+                splitk_mfma<MODE>(a, b, p1, p2, p3);
             }
         }
     }
+
+    floatx16 cre, cim;
+    combine3<MODE>(p1, p2, p3, cre, cim);  // linear: partial sums combine like whole ones
 
     if constexpr (SK == 1) {
         if (!live) return;

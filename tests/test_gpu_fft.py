@@ -33,6 +33,8 @@ CASES = [
     (32, 3, 27, 27, 2, 2), (32, 48, 32, 32, 0, 0), (32, 17, 5, 5, 0, 0), (32, 35, 20, 28, 5, 1),
     (64, 9, 55, 55, 4, 4), (64, 16, 64, 64, 0, 0), (64, 5, 9, 9, 0, 0), (64, 11, 33, 40, 7, 10),
     (64, 19, 16, 16, 0, 0), (64, 3, 1, 16, 0, 0), (64, 8, 11, 2, 0, 0), (64, 4, 9, 9, 1, 0),   # small planes: zero inputs skipped
+    (64, 37, 47, 47, 0, 0), (64, 50, 21, 35, 3, 5), (64, 41, 9, 9, 0, 0), (32, 70, 27, 27, 2, 2), (16, 200, 13, 13, 1, 1),   # several workgroups, ragged last one
+    (64, 23, 63, 63, 1, 1), (64, 18, 1, 63, 63, 0), (32, 19, 31, 1, 0, 31),   # planes that touch the canvas border
     (128, 5, 100, 100, 3, 7), (128, 9, 128, 128, 0, 0), (128, 6, 11, 11, 0, 0), (128, 3, 70, 127, 20, 1),
 ]
 
