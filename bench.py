@@ -66,9 +66,9 @@ def stage_model(cfg, pass_, n, q):
 # (profiles/hbm_traffic_all_configs.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, the
 # factors a 256 MiB device copy gives for the same counters (--calibrate-copy).
 MEASURED_TRAFFIC_MAIN = {
-    "cgemm_hybrid_kernel<0>": (17087 * 2.0 + 16640) * 1024,
-    "cgemm_hybrid_kernel<1>": (17088 * 2.0 + 16640) * 1024,
-    "cgemm_hybrid_kernel<2>": (17087 * 2.0 + 16640) * 1024,
+    "cgemm_hybrid_kernel<0>": (17091 * 2.0 + 16642) * 1024,
+    "cgemm_hybrid_kernel<1>": (17096 * 2.0 + 16642) * 1024,
+    "cgemm_hybrid_kernel<2>": (17096 * 2.0 + 16641) * 1024,
 }
 
 KERNEL_OF_STAGE = {"fft": "rfft2d_kernel", "mm": "cgemm_freq_kernel", "ifft": "irfft2d_kernel"}
