@@ -7,17 +7,16 @@
 // 0, 1, 2 below.  Operands are frequency-major, so each frequency is a dense
 // row-major complex matrix and no transpose kernel exists.
 //
-// A complex product is carried as a real GEMM with doubled inner dimension:
-//   C_re = sum_k' A'[m][k'] Bre'[k'][n],  C_im = sum_k' A'[m][k'] Bim'[k'][n]
-// where k' enumerates (k, re|im).  A' is the interleaved storage read as it
-// lies; Bre'/Bim' are B with its components swapped and sign-flipped in
-// registers.  v_mfma_f32_32x32x2_f32 takes the two k' of a step from the two
-// half-waves; because a sum may run over k' in any order, each half-wave is
-// given the k' that are contiguous for it in LDS.
+// v_mfma_f32_32x32x2_f32 takes the two k of a step from the two half-waves; because a
+// sum may run over k in any order, each half-wave is given the k that are contiguous for
+// it in memory.  The MFMA kernels form a complex product from three real ones (cmac3
+// below); the bounds-checked general kernel carries it as a real GEMM with doubled inner
+// dimension, C_re = sum_k' A'[m][k'] Bre'[k'][n], C_im = sum_k' A'[m][k'] Bim'[k'][n] with
+// k' = (k, re|im), A' the interleaved storage as it lies and Bre'/Bim' B with its
+// components swapped and sign-flipped in registers.
 //
-// Workgroup: 256 lanes = 4 waves in 2x2, each wave a 32x32 complex block
-// (2 x 16 accumulator registers); tile 64 x 64 x 16 complex per step with
-// register-prefetch double buffering through LDS.
+// Workgroup of the general kernel: 256 lanes = 4 waves in 2x2, each wave a 32x32 complex
+// block; tile 64 x 64 x 16 complex per step with register-prefetch double buffering through LDS.
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>

@@ -1,11 +1,11 @@
-// Batched 2-D real<->complex FFT kernels for gfx950 (power-of-two N, 8..64).
+// Batched 2-D real<->complex FFT kernels for gfx950 (power-of-two N, 8..128).
 //
 // Replaces what the reference asks of fbcuda's fbfft2D / fbifft2D through
 // src/fft/FBFFTHost.cpp:39-116 (call sites :86-88, :93, :101-111): implicit zero
 // padding at (padU, padL) on the way in, crop at (padU, padL) on the way out,
 // Hermitian half spectrum, unnormalised inverse.
 //
-// Design (one workgroup = T consecutive planes, T*N/2 = 256 lanes):
+// Design (one workgroup = T consecutive planes, T*N/2 lanes: 256, or 512 for N = 64):
 //   * the T planes are one contiguous chunk of the real tensor: it is copied to
 //     LDS with fully coalesced loads;
 //   * row pass: one lane transforms TWO real rows at once as one complex
@@ -13,8 +13,7 @@
 //     the two Hermitian spectra; columns 0 and N/2 of a real row spectrum are
 //     real, so they share one complex slot and the tile is exactly N/2 wide;
 //   * the tile R[y][kx][t] (plane index t fastest) lives in LDS, aliasing the
-//     staging chunk; rows of the canvas that are known to be zero are neither
-//     stored nor read back;
+//     staging chunk; every canvas row has its fixed place in it;
 //   * column pass: one lane transforms one column (N complex points) in
 //     registers; the lane owning slot 0 untangles columns 0 and N/2;
 //   * results go straight from registers to the frequency-major buffer
