@@ -195,9 +195,9 @@ def measure_config(nn, torch, synth, name, steps, warmup):
                 ach = spec[1] / (ms_s * 1e-3) / 1e12
                 mnk = {"fprop": (B, F, P), "bprop": (B, P, F), "accgrad": (F, P, B)}[p]
                 kname = mm_kernel_name(p, q - (n - 2), *mnk)
-                # the MFMA kernels form a complex product from three real ones: they issue 6 of the
-                # 8 algorithmic flops per complex multiply-add (the bounds-checked general kernel: all 8)
-                issued = spec[1] * (1.0 if kname.startswith("cgemm_freq_kernel") else 0.75)
+                # the kernels form a complex product from three real ones: they issue 6 of the
+                # 8 algorithmic flops per complex multiply-add
+                issued = spec[1] * 0.75
                 entry["stages"][s] = {"kernel": kname, "ms": ms_s, "bound": "mfma",
                                       "flops": spec[1], "bytes": spec[2], "achieved": ach,
                                       "unit": "TFLOP/s", "peak": MFMA_FP32_PEAK_TF,

@@ -9,11 +9,7 @@
 //
 // v_mfma_f32_32x32x2_f32 takes the two k of a step from the two half-waves; because a
 // sum may run over k in any order, each half-wave is given the k that are contiguous for
-// it in memory.  The MFMA kernels form a complex product from three real ones (cmac3
-// below); the bounds-checked general kernel carries it as a real GEMM with doubled inner
-// dimension, C_re = sum_k' A'[m][k'] Bre'[k'][n], C_im = sum_k' A'[m][k'] Bim'[k'][n] with
-// k' = (k, re|im), A' the interleaved storage as it lies and Bre'/Bim' B with its
-// components swapped and sign-flipped in registers.
+// it in memory.  A complex product is formed from three real ones (cmac3 below).
 //
 // Workgroup of the general kernel: 256 lanes = 4 waves in 2x2, each wave a 32x32 complex
 // block; tile 64 x 64 x 16 complex per step with register-prefetch double buffering through LDS.
@@ -73,6 +69,39 @@ __device__ __forceinline__ void store_tile(float *lds, int tid, const float2 (&v
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Complex products with three real MFMAs instead of four.  With
+//   P1 = sum ar br,  P2 = sum ai bi,  P3 = sum (ar +- ai)(br +- bi)
+// the three modes are
+//   A conj(B):     Re = P1 + P2,  Im = P3 - P1 + P2,  P3 from (ar + ai)(br - bi)
+//   A B:           Re = P1 - P2,  Im = P3 - P1 - P2,  P3 from (ar + ai)(br + bi)
+//   conj(A)^T B:   Re = P1 + P2,  Im = P3 - P1 + P2,  P3 from (ar - ai)(br + bi)
+// i.e. 6 instead of 8 flops per complex multiply-add on the matrix cores, paid for with two
+// vector adds per operand element and a third accumulator (16 registers per 32x32 block).
+// ---------------------------------------------------------------------------------------
+template <int MODE>
+__device__ __forceinline__ void cmac3(float ar, float ai, float br, float bi, floatx16 &p1, floatx16 &p2,
+                                      floatx16 &p3)
+{
+    const float sa = (MODE == 2) ? ar - ai : ar + ai;
+    const float sb = (MODE == 0) ? br - bi : br + bi;
+    p1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, p1, 0, 0, 0);
+    p2 = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, bi, p2, 0, 0, 0);
+    p3 = __builtin_amdgcn_mfma_f32_32x32x2f32(sa, sb, p3, 0, 0, 0);
+}
+
+template <int MODE>
+__device__ __forceinline__ void combine3(const floatx16 &p1, const floatx16 &p2, const floatx16 &p3,
+                                         floatx16 &cre, floatx16 &cim)
+{
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const float s2 = (MODE == 1) ? -p2[r] : p2[r];
+        cre[r] = p1[r] + s2;
+        cim[r] = (p3[r] - p1[r]) + s2;
+    }
+}
+
 template <int MODE>
 __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restrict__ A,
                                                          const float2 *__restrict__ B,
@@ -106,9 +135,9 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
     const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 31, h = lane >> 5;
 
-    floatx16 cre, cim;
+    floatx16 p1, p2, p3;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { cre[r] = 0.f; cim[r] = 0.f; }
+    for (int r = 0; r < 16; ++r) { p1[r] = 0.f; p2[r] = 0.f; p3[r] = 0.f; }
 
     float2 pa[4], pb[4];
     const int nk = (K + KT - 1) / KT;
@@ -149,13 +178,7 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
                 b[4 * j] = vb.x; b[4 * j + 1] = vb.y; b[4 * j + 2] = vb.z; b[4 * j + 3] = vb.w;
             }
 #pragma unroll
-            for (int s = 0; s < 16; s += 2) {
-                // k' = (k, re): A' = a_re ; k' = (k, im): A' = a_im.   C = A conj(B)
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], -b[s + 1], cim, 0, 0, 0);
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s + 1], b[s + 1], cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s + 1], b[s], cim, 0, 0, 0);
-            }
+            for (int s = 0; s < 16; s += 2) cmac3<0>(a[s], a[s + 1], b[s], b[s + 1], p1, p2, p3);  // C = A conj(B)
         } else if (MODE == 1) {
             // A K-contiguous (as above); B row-contiguous [k][n]: one (re,im) pair per two steps
             float a[16];
@@ -167,23 +190,15 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
 #pragma unroll
             for (int kk = 0; kk < 8; ++kk) {
                 const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDM + 2 * bcol);
-                // C = A B
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.x, cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk], vb.y, cim, 0, 0, 0);
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], -vb.y, cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2 * kk + 1], vb.x, cim, 0, 0, 0);
+                cmac3<1>(a[2 * kk], a[2 * kk + 1], vb.x, vb.y, p1, p2, p3);  // C = A B
             }
         } else {
-            // both row-contiguous [k][.]: step s is complex k = s; half-wave 0 feeds the real
-            // part of A, half-wave 1 the imaginary part.   C = conj(A)^T B
+            // both row-contiguous [k][.]: half-wave h owns k = 8h + kk.   C = conj(A)^T B
 #pragma unroll
-            for (int s = 0; s < KT; ++s) {
-                const float av = as[s * LDM + 2 * arow + h];
-                const float2 vb = *reinterpret_cast<const float2 *>(bs + s * LDM + 2 * bcol);
-                const float opre = h ? vb.y : vb.x;
-                const float opim = h ? -vb.x : vb.y;
-                cre = __builtin_amdgcn_mfma_f32_32x32x2f32(av, opre, cre, 0, 0, 0);
-                cim = __builtin_amdgcn_mfma_f32_32x32x2f32(av, opim, cim, 0, 0, 0);
+            for (int kk = 0; kk < 8; ++kk) {
+                const float2 va = *reinterpret_cast<const float2 *>(as + (8 * h + kk) * LDM + 2 * arow);
+                const float2 vb = *reinterpret_cast<const float2 *>(bs + (8 * h + kk) * LDM + 2 * bcol);
+                cmac3<2>(va.x, va.y, vb.x, vb.y, p1, p2, p3);
             }
         }
 
@@ -194,6 +209,8 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
     }
 
     // epilogue: accumulator register r of lane (li, h) is C[8*(r/4) + 4*h + r%4][li] of the block
+    floatx16 cre, cim;
+    combine3<MODE>(p1, p2, p3, cre, cim);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int row = m0 + 32 * wm + 8 * (r / 4) + 4 * h + (r % 4);
@@ -208,39 +225,6 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
             }
             store_nt(dst, v);
         }
-    }
-}
-
-// ---------------------------------------------------------------------------------------
-// Complex products with three real MFMAs instead of four.  With
-//   P1 = sum ar br,  P2 = sum ai bi,  P3 = sum (ar +- ai)(br +- bi)
-// the three modes are
-//   A conj(B):     Re = P1 + P2,  Im = P3 - P1 + P2,  P3 from (ar + ai)(br - bi)
-//   A B:           Re = P1 - P2,  Im = P3 - P1 - P2,  P3 from (ar + ai)(br + bi)
-//   conj(A)^T B:   Re = P1 + P2,  Im = P3 - P1 + P2,  P3 from (ar - ai)(br + bi)
-// i.e. 6 instead of 8 flops per complex multiply-add on the matrix cores, paid for with two
-// vector adds per operand element and a third accumulator (16 registers per 32x32 block).
-// ---------------------------------------------------------------------------------------
-template <int MODE>
-__device__ __forceinline__ void cmac3(float ar, float ai, float br, float bi, floatx16 &p1, floatx16 &p2,
-                                      floatx16 &p3)
-{
-    const float sa = (MODE == 2) ? ar - ai : ar + ai;
-    const float sb = (MODE == 0) ? br - bi : br + bi;
-    p1 = __builtin_amdgcn_mfma_f32_32x32x2f32(ar, br, p1, 0, 0, 0);
-    p2 = __builtin_amdgcn_mfma_f32_32x32x2f32(ai, bi, p2, 0, 0, 0);
-    p3 = __builtin_amdgcn_mfma_f32_32x32x2f32(sa, sb, p3, 0, 0, 0);
-}
-
-template <int MODE>
-__device__ __forceinline__ void combine3(const floatx16 &p1, const floatx16 &p2, const floatx16 &p3,
-                                         floatx16 &cre, floatx16 &cim)
-{
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const float s2 = (MODE == 1) ? -p2[r] : p2[r];
-        cre[r] = p1[r] + s2;
-        cim[r] = (p3[r] - p1[r]) + s2;
     }
 }
 
