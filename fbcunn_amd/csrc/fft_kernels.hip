@@ -31,7 +31,7 @@ namespace fbfc {
 
 // SMALL: the forward variant for planes of at most 16 x 16 at N = 64: its tile has so few rows that
 // all columns fit at once, so it runs in one phase (144 -> 137 us for 24576 planes of 9 x 9).
-template <int N, bool INVERSE = false, bool SMALL = false>
+template <int N, bool INVERSE = false, bool SMALL = false, int PHASES = 0>
 struct FftShape {
     // planes per workgroup: 256 lanes' worth, except N = 64, which takes 16 planes (512 lanes) so
     // that its runs per frequency are whole 128-byte lines -- measured with the bare
@@ -47,7 +47,8 @@ struct FftShape {
     // Phases: the LDS tile holds NH2/PH of the tile columns at a time and the input /
     // output staging area T/PH planes at a time, so that two workgroups fit one CU's
     // 160 KB LDS even for N = 64 (a full 8-plane tile would need 117 KB).
-    static constexpr int PH = SMALL ? 1 : (N >= 128) ? 4 : (N >= 64) ? 2 : (N == 32 && !INVERSE) ? 2 : 1;
+    // PHASES > 0 overrides the choice (the N = 32 inverse of many planes, see launch_inv)
+    static constexpr int PH = PHASES > 0 ? PHASES : SMALL ? 1 : (N >= 128) ? 4 : (N >= 64) ? 2 : (N == 32 && !INVERSE) ? 2 : 1;
     static constexpr int KXP = NH2 / PH;    // tile columns per phase
     static constexpr int TP = T / PH;       // planes per staging round
     // waves per SIMD the register budget is sized for (N = 128 keeps 256 values per lane)
@@ -540,15 +541,15 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
 // inverse: freq [N*(N/2+1)][planes] complex -> real (planes,h,w), unnormalised,
 // real[r][s] = y[r+padU][s+padL] (+ bias[plane % bias_period])
 // ---------------------------------------------------------------------------------
-template <int N, bool WIN>
-__global__ __launch_bounds__((FftShape<N, true>::THREADS), (FftShape<N, true>::MIN_WAVES)) void irfft2d_kernel(const float2 *__restrict__ in,
+template <int N, bool WIN, int PHASES = 0>
+__global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftShape<N, true, false, PHASES>::MIN_WAVES)) void irfft2d_kernel(const float2 *__restrict__ in,
                                                       float *__restrict__ out, long planes,
                                                       int h, int w, int padU, int padL,
                                                       const float *__restrict__ bias,
                                                       int bias_period, int vec4, BiasGradJob bgrad,
                                                       unsigned bgrad_blocks, Window win, int tbl_off)
 {
-    using S = FftShape<N, true>;
+    using S = FftShape<N, true, false, PHASES>;
     constexpr int T = S::T;
     extern __shared__ __align__(16) float smem[];
     if (blockIdx.x < bgrad_blocks) {
@@ -694,10 +695,10 @@ __global__ __launch_bounds__((FftShape<N, true>::THREADS), (FftShape<N, true>::M
 // ---------------------------------------------------------------------------------
 // host launchers
 // ---------------------------------------------------------------------------------
-template <int N, bool INVERSE, bool SMALL = false>
+template <int N, bool INVERSE, bool SMALL = false, int PHASES = 0>
 static size_t fft_lds_bytes(int h, int w, int padU)
 {
-    using S = FftShape<N, INVERSE, SMALL>;
+    using S = FftShape<N, INVERSE, SMALL, PHASES>;
     (void)padU;
     // the tile holds every canvas row at a fixed place (the rows the small-plane forward variant reads)
     const size_t tile = (size_t)(SMALL ? 16 : N) * S::ROWSTRIDE * sizeof(float2);
@@ -785,18 +786,18 @@ static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_
     return launch_fwd_impl<N, WIN, NZ, false>(a, second, s);
 }
 
-template <int N, bool WIN>
-static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
+template <int N, bool WIN, int PHASES>
+static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s)
 {
-    using S = FftShape<N, true>;
+    using S = FftShape<N, true, false, PHASES>;
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&irfft2d_kernel<N, WIN>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&irfft2d_kernel<N, WIN, PHASES>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    size_t lds = fft_lds_bytes<N, true>(a.h, a.w, a.padU);
+    size_t lds = fft_lds_bytes<N, true, false, PHASES>(a.h, a.w, a.padU);
     const int tbl_off = (int)(lds / sizeof(float));
     if (WIN) lds += S::T * sizeof(int4);
     long blocks = (a.planes + S::T - 1) / S::T;
@@ -806,10 +807,22 @@ static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
                                a.out_planes};
     const unsigned bblocks = (bgrad.dc != nullptr) ? bias_grad_dc_blocks(bgrad.planes) : 0u;
     if (blocks + bblocks > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((irfft2d_kernel<N, WIN>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
+    hipLaunchKernelGGL((irfft2d_kernel<N, WIN, PHASES>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
                        reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL,
                        a.bias, a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks, a.win, tbl_off);
     return hipGetLastError();
+}
+
+template <int N, bool WIN>
+static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
+{
+    // N = 32: with the whole tile in LDS two workgroups share a CU, in two phases four do.  A launch
+    // of more than two rounds of workgroups is faster with the four (65536 planes of 27 x 27: 95 ->
+    // 84 us), a launch of one round with the whole tile (8192 planes of 27 x 27: 11.3 against 12.1 us).
+    if constexpr (N == 32) {
+        if (a.planes > 2L * 512 * FftShape<N, true>::T) return launch_inv_impl<N, WIN, 2>(a, s);
+    }
+    return launch_inv_impl<N, WIN, 0>(a, s);
 }
 
 // the kernels address a frequency row with 32-bit lane offsets

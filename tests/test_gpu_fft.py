@@ -82,6 +82,20 @@ def test_inverse_matches_idft(nn, oracle, n, planes, h, w, pu, pl):
     assert np.abs(got[pick] - o).max() <= TOL * np.abs(want).max() * 4
 
 
+def test_inverse_n32_many_planes(nn):
+    """More than two rounds of workgroups: the N = 32 inverse switches to its two-phase variant."""
+    n, distinct, reps, h, w, pu, pl = 32, 129, 130, 27, 25, 2, 3
+    full = synth.uniform(77, (distinct, n, n))
+    spec = np.tile(np.fft.rfft2(full.astype(np.float64)), (reps, 1, 1))
+    planes = distinct * reps
+    out = torch.full((planes, h, w), float("nan"), device="cuda")
+    nn.FFTWrapper("fbfft", pl, pu).ffti(out, dev(planes_to_freq_major(spec)))
+    got = host(out)
+    want = np.tile(full[:, pu:pu + h, pl:pl + w].astype(np.float64) * (n * n), (reps, 1, 1))
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL * np.abs(want).max() * 4
+
+
 def test_inverse_adds_bias_per_plane(nn):
     n, B, F, h = 16, 3, 5, 13
     full = synth.uniform(31, (B * F, n, n))
