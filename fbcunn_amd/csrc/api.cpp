@@ -235,6 +235,7 @@ fbfc::Window make_window(int d1, int nty, int ntx, int step_y, int step_x, int o
     w.off_x = off_x;
     w.img_h = img_h;
     w.img_w = img_w;
+    w.remap = 0;  // decided per launch
     return w;
 }
 

@@ -63,6 +63,30 @@ struct FftShape {
     static constexpr int LPR = THREADS / PH;
 };
 
+// Windowed operands: virtual plane v = (b * nt + tile) * d1 + c, so the workgroups of one tile (d1 / T of
+// them) are followed by those of the next tile -- on other XCDs, although neighbouring windows of one
+// image plane share cache lines (a 128-byte window row at an arbitrary offset touches two lines).  With
+// remap set, launch index j = 8 r + x is given group u = 8 (r / nt) + x of the d0 * d1 / T (batch, plane
+// group) pairs and tile r % nt: XCD x walks through the tiles of its groups one after the other, and the
+// shared lines are still in its L2.  Needs d1 % T == 0 and (d0 * d1 / T) % 8 == 0.
+template <int T>
+__device__ __forceinline__ long window_block(unsigned j, const Window &w)
+{
+    const unsigned G = (unsigned)w.d1 / T, nt = (unsigned)w.nt;
+    const unsigned x = j & 7u, r = j >> 3;
+    const unsigned tile = r % nt, u = (r / nt) * 8u + x;
+    const unsigned b = u / G, cg = u - b * G;
+    return (long)(b * nt + tile) * G + cg;
+}
+
+template <int T>
+static int window_remap_ok(const Window &w, long planes)
+{
+    if (!w.on || w.d1 % T != 0) return 0;
+    const long groups = planes / ((long)w.nt * w.d1) * (w.d1 / T);
+    return groups % 8 == 0 && planes / T < (1L << 31);
+}
+
 // LDS staging area in canvas-row layout.  Row (p*h + r) of the staged planes starts at
 // (p*h + r) * LDR floats and holds the N canvas columns of that row: input column x sits
 // at padL + x, the margins are zero.  LDR = N + 4 floats keeps rows 16-byte aligned (the
@@ -328,11 +352,14 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
     const int padU = second ? job1.padU : job0.padU, padL = second ? job1.padL : job0.padL;
     const int vec4 = second ? job1.vec4 : job0.vec4;
     const int herm = second ? job1.herm : job0.herm;
-    const long x0 = plane_group<T>(v - (second ? blocks0 : 0u)) * T;
+    [[maybe_unused]] const Window &win = second ? job1.win : job0.win;
+    long x0 = plane_group<T>(v - (second ? blocks0 : 0u)) * T;
+    if constexpr (WIN) {
+        if (win.remap) x0 = window_block<T>(v - (second ? blocks0 : 0u), win) * T;
+    }
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
-    [[maybe_unused]] const Window &win = second ? job1.win : job0.win;
     [[maybe_unused]] int4 *tbl = reinterpret_cast<int4 *>(smem + (second ? job1.tbl_off : job0.tbl_off));
     if constexpr (WIN) {
         if (win.on) build_window_table<N>(tbl, win, x0, planes, tid);
@@ -559,7 +586,10 @@ __global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftSh
         return;
     }
     const int tid = threadIdx.x;
-    const long x0 = plane_group<T>(blockIdx.x - bgrad_blocks) * T;
+    long x0 = plane_group<T>(blockIdx.x - bgrad_blocks) * T;
+    if constexpr (WIN) {
+        if (win.remap) x0 = window_block<T>(blockIdx.x - bgrad_blocks, win) * T;
+    }
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
@@ -732,6 +762,7 @@ static FwdJob make_job(const FwdArgs &a)
     j.tbl_off = 0;
     j.herm = a.herm;
     j.win = a.win;
+    j.win.remap = window_remap_ok<S::T>(a.win, a.planes);
     return j;
 }
 
@@ -803,13 +834,15 @@ static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s)
     long blocks = (a.planes + S::T - 1) / S::T;
     if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
     const int vec4 = ((reinterpret_cast<uintptr_t>(a.out) & 15) == 0) && (((long)S::T * a.h * a.w) % 4 == 0);
+    Window win = a.win;
+    win.remap = window_remap_ok<S::T>(a.win, a.planes);
     const BiasGradJob bgrad = {reinterpret_cast<const float2 *>(a.go_freq), a.grad_bias, a.scale, a.batch,
                                a.out_planes};
     const unsigned bblocks = (bgrad.dc != nullptr) ? bias_grad_dc_blocks(bgrad.planes) : 0u;
     if (blocks + bblocks > 0x7fffffffL) return hipErrorInvalidValue;
     hipLaunchKernelGGL((irfft2d_kernel<N, WIN, PHASES>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
                        reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL,
-                       a.bias, a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks, a.win, tbl_off);
+                       a.bias, a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks, win, tbl_off);
     return hipGetLastError();
 }
 

@@ -16,6 +16,7 @@ hipError_t launch_rfft2d(int N, const float *in, float *out, long planes, int h,
 struct Window {
     int on;
     int d1, nt, ntx, step_y, step_x, off_y, off_x, img_h, img_w;
+    int remap;  // set by the launchers: workgroups walk the tiles of one plane group on one XCD
 };
 // Two forward transforms of the same size in one launch (the two FFTs of a pass).
 struct FwdArgs {
