@@ -42,13 +42,13 @@ struct FftShape {
     static constexpr int THREADS = T * N / 2;
     static constexpr int NH2 = N / 2;       // complex slots per tile row
     static constexpr int NH = N / 2 + 1;    // stored column frequencies
-    // (N = 32 forward: two phases halve the LDS footprint and a third workgroup fits a CU, measured
-    // 19.6 -> 17.4 us for config 3's pair of transforms; the inverse was slower that way and keeps one.)
-    // Phases: the LDS tile holds NH2/PH of the tile columns at a time and the input /
-    // output staging area T/PH planes at a time, so that two workgroups fit one CU's
-    // 160 KB LDS even for N = 64 (a full 8-plane tile would need 117 KB).
+    // Phases: the LDS tile holds NH2/PH of the tile columns at a time (the others wait in registers)
+    // and the input / output staging area T/PH planes at a time.  N >= 64: two phases, a whole tile
+    // would not fit the 160 KB of LDS (N = 128 ran in four until the waiting columns made it spill).
+    // N = 32 forward: two phases halve the LDS footprint and a third workgroup fits a CU, measured
+    // 19.6 -> 17.4 us for config 3's pair of transforms; the inverse keeps one unless the launch is large.
     // PHASES > 0 overrides the choice (the N = 32 inverse of many planes, see launch_inv)
-    static constexpr int PH = PHASES > 0 ? PHASES : SMALL ? 1 : (N >= 128) ? 4 : (N >= 64) ? 2 : (N == 32 && !INVERSE) ? 2 : 1;
+    static constexpr int PH = PHASES > 0 ? PHASES : SMALL ? 1 : (N >= 64) ? 2 : (N == 32 && !INVERSE) ? 2 : 1;
     static constexpr int KXP = NH2 / PH;    // tile columns per phase
     static constexpr int TP = T / PH;       // planes per staging round
     // waves per SIMD the register budget is sized for (N = 128 keeps 256 values per lane)
