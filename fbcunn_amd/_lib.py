@@ -58,12 +58,16 @@ SIGNATURES = {
     "fbfc_plan_set_reuse": (_i, [_vp, ctypes.c_uint]),
     "fbfc_plan_set_timed": (_i, [_vp, _i]),
     "fbfc_plan_stage_ms": (_i, [_vp, ctypes.POINTER(_f), _i]),
+    "fbfc_plan_contraction_kernel": (_i, [_vp, ctypes.c_char_p, ctypes.c_size_t]),
+    "fbfc_debug_force_contraction_kernel": (_i, [_i]),
     "fbfc_fft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp]),
     "fbfc_ifft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
     "fbfc_fft1d": (_i, [_vp, _l, _i, _i, _i, _vp, _vp]),
     "fbfc_ifft1d": (_i, [_vp, _l, _i, _i, _i, _vp, _vp]),
     "fbfc_transpose_mm": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _vp]),
     "fbfc_update_output_bias": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
+    "fbfc_update_output_bias_strided": (_i, [_vp, _vp, _i, _i, _i, _i, _l, _l, _l, _l, _l, _vp]),
+    "fbfc_acc_grad_parameters_bias_strided": (_i, [_vp, _vp, _f, _i, _i, _i, _i, _l, _l, _l, _l, _l, _vp, _vp]),
     "fbfc_bias_grad_scratch_bytes": (ctypes.c_size_t, [_i, _i]),
     "fbfc_acc_grad_parameters_bias": (_i, [_vp, _vp, _f, _i, _i, _i, _i, _vp, _vp]),
 }

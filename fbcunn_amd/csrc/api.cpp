@@ -43,6 +43,29 @@ int next_power_of_2(int v)
 
 int imax(int a, int b) { return a > b ? a : b; }
 
+// One launch transforms all planes of a tensor and addresses a frequency row of its spectrum with
+// 32-bit byte offsets: batch * tiles * planes (and out_planes * in_planes) must stay below
+// fft_max_planes(n).  Checked when the plan is made, so that an oversized layer is refused with the
+// numbers in the message instead of failing at its first pass.
+int planes_limit(int n, long batch, long tiles, long in_planes, long out_planes)
+{
+    const long lim = fbfc::fft_max_planes(n);
+    const long vb = batch * tiles;  // at most 2^31 * 2^31: no overflow in long
+    const long cand[3] = {vb * in_planes, vb * out_planes, out_planes * in_planes};
+    const char *what[3] = {"batch x tiles x input planes", "batch x tiles x output planes",
+                           "output planes x input planes"};
+    for (int i = 0; i < 3; ++i) {
+        if (vb > lim || cand[i] > lim) {
+            char buf[200];
+            std::snprintf(buf, sizeof buf,
+                          "%s = %ld planes exceed the %ld one FFT of size %d can take in a launch "
+                          "(split the batch)", what[i], cand[i], lim, n);
+            return fail(FBFC_ERR_UNSUPPORTED_SIZE, buf);
+        }
+    }
+    return FBFC_OK;
+}
+
 int plan_query(const fbfc_conv_desc *d, fbfc_plan_info *info)
 {
     if (d == nullptr || info == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
@@ -70,6 +93,8 @@ int plan_query(const fbfc_conv_desc *d, fbfc_plan_info *info)
         std::snprintf(buf, sizeof buf, "FFT size %d not supported (8..%d)", n, kMaxFft);
         return fail(FBFC_ERR_UNSUPPORTED_SIZE, buf);
     }
+    const int lim = planes_limit(n, d->batch, 1, d->in_planes, d->out_planes);
+    if (lim != FBFC_OK) return lim;
     const size_t q = (size_t)n * (n / 2 + 1);
     info->fft_size = n;
     info->n_freq = (int)q;
@@ -122,6 +147,8 @@ int plan_query_tiled(const fbfc_conv_desc *d, int tile_h, int tile_w, fbfc_plan_
     const size_t nt_out = (size_t)ceil_div(out_h, step_h) * ceil_div(out_w, step_w);
     const size_t nt_in = (size_t)ceil_div(d->in_h, step_h) * ceil_div(d->in_w, step_w);
     const size_t nt = nt_out > nt_in ? nt_out : nt_in;
+    const int lim = planes_limit(n, d->batch, (long)nt, d->in_planes, d->out_planes);
+    if (lim != FBFC_OK) return lim;
     info->fft_size = n;
     info->n_freq = (int)q;
     info->out_h = out_h;
@@ -164,6 +191,7 @@ struct fbfc_plan {
     hipEvent_t ev[FBFC_NUM_STAGES + 1];
     bool ev_made;
     float stage_ms[FBFC_NUM_STAGES];
+    char mm_kernel[48];  // the contraction kernel the last pass launched
 };
 
 namespace {
@@ -317,6 +345,7 @@ static int plan_create(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_
     p->tiled = tiled;
     set_geometry(p, tile_h, tile_w);
     hipError_t e = hipGetDevice(&p->device);
+    if (e == hipSuccess) e = fbfc::fft_prepare_device();
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->in_freq), info.input_freq_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->w_freq), info.weight_freq_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->out_freq), info.output_freq_bytes);
@@ -394,6 +423,21 @@ int fbfc_plan_set_timed(fbfc_plan *p, int on)
     return FBFC_OK;
 }
 
+int fbfc_plan_contraction_kernel(const fbfc_plan *p, char *name, size_t n)
+{
+    if (p == nullptr || name == nullptr || n == 0) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    std::snprintf(name, n, "%s", p->mm_kernel);
+    return FBFC_OK;
+}
+
+int fbfc_debug_force_contraction_kernel(int variant)
+{
+    if (variant != -1 && variant != 0 && variant != 1 && variant != 2 && variant != 4 && variant != 8 && variant != 9)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "contraction kernel variant must be -1, 0, 1, 2, 4, 8 or 9");
+    fbfc::cgemm_force_variant(variant);
+    return FBFC_OK;
+}
+
 int fbfc_plan_stage_ms(const fbfc_plan *p, float *ms, int n)
 {
     if (p == nullptr || ms == nullptr || n < 0) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
@@ -431,10 +475,13 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     p->have_in = true;
     p->have_w = true;
     float *res = p->reuse ? p->res_freq : p->out_freq;
-    if (!p->reuse) p->have_out = false;
+    // a new forward pass starts a new step: a spectrum of gradOutput left in the plan belongs to
+    // the previous one, whatever the reuse policy
+    p->have_out = false;
     // O[b][f] = 1/N^2 sum_p I[b][p] conj(W[f][p])   (SpatialConvolutionFBFFT.lua:157-164)
     FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(0, p->in_freq, p->w_freq, res, QH, fm, g.vbatch, d.out_planes,
                                      d.in_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(fprop)");
+    std::snprintf(p->mm_kernel, sizeof p->mm_kernel, "%s", fbfc::cgemm_last_kernel());
     tm.done(FBFC_STAGE_MM);
     const fbfc::InvArgs inv = {res, output, (long)g.vbatch * d.out_planes, g.r_h, g.r_w, g.r_pad_u, g.r_pad_l,
                                bias, d.out_planes, g.r_win, nullptr, nullptr, 0.0f, 0, 0};
@@ -475,6 +522,7 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     // GI[b][p] = 1/N^2 sum_f GO[b][f] W[f][p]   (SpatialConvolutionFBFFT.lua:244-251)
     FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(1, p->out_freq, p->w_freq, res, QH, fm, g.vbatch, d.in_planes,
                                      d.out_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(bprop)");
+    std::snprintf(p->mm_kernel, sizeof p->mm_kernel, "%s", fbfc::cgemm_last_kernel());
     tm.done(FBFC_STAGE_MM);
     const fbfc::InvArgs inv = {res, grad_input, (long)g.vbatch * d.in_planes, g.r_h, g.r_w, g.r_pad_u,
                                g.r_pad_l, nullptr, 1, g.r_win, nullptr, nullptr, 0.0f, 0, 0};
@@ -515,13 +563,13 @@ static int acc_grad_parameters(fbfc_plan *p, const float *input, const float *gr
         FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fin, s), "rfft2d(input)");
         tm.done(FBFC_STAGE_FFT_B);
     }
-    p->have_out = true;
     p->have_in = true;
     float *res = p->reuse ? p->res_freq : p->w_freq;
     if (!p->reuse) p->have_w = false;
     // GW[f][p] = scale/N^2 sum_b conj(GO[b][f]) I[b][p]   (SpatialConvolutionFBFFT.lua:337-344)
     FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(2, p->out_freq, p->in_freq, res, QH, fm, d.out_planes, d.in_planes,
                                      g.vbatch, scale / ((float)N * (float)N), 0, s), "cgemm(accGrad)");
+    std::snprintf(p->mm_kernel, sizeof p->mm_kernel, "%s", fbfc::cgemm_last_kernel());
     tm.done(FBFC_STAGE_MM);
     fbfc::InvArgs inv = {res, grad_weight, (long)d.out_planes * d.in_planes, g.r_h, g.r_w, 0, 0, nullptr, 1, {},
                          nullptr, nullptr, 0.0f, 0, 0};
@@ -536,6 +584,9 @@ static int acc_grad_parameters(fbfc_plan *p, const float *input, const float *gr
     }
     FBFC_STAGE(tm, fbfc::launch_irfft2d_args(N, inv, s), "irfft2d(gradWeight) + bias grad");
     tm.done(FBFC_STAGE_IFFT);
+    // the spectrum of gradOutput is good for the accGradParameters that follows the updateGradInput
+    // of the same gradOutput, once: a second accGradParameters transforms its own
+    p->have_out = false;
     return tm.finish();
 }
 
@@ -564,6 +615,7 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
     if (planes < 1 || h < 1 || w < 1 || pad_u < 0 || pad_l < 0 || h + pad_u > fft_size ||
         w + pad_l > fft_size)
         return fail(FBFC_ERR_INVALID_ARGUMENT, "plane plus padding must fit the FFT size");
+    FBFC_TRY(fbfc::fft_prepare_device(), "device set-up");
     if (fft_size_tiny(fft_size)) {
         FBFC_TRY(fbfc::launch_rfft2d_tiny(fft_size, real, freq, planes, h, w, pad_u, pad_l,
                                           static_cast<hipStream_t>(stream)), "rfft2d");
@@ -584,6 +636,7 @@ int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad
         w + pad_l > fft_size)
         return fail(FBFC_ERR_INVALID_ARGUMENT, "plane plus padding must fit the FFT size");
     if (bias != nullptr && bias_period < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "bias_period must be positive");
+    FBFC_TRY(fbfc::fft_prepare_device(), "device set-up");
     if (fft_size_tiny(fft_size)) {
         FBFC_TRY(fbfc::launch_irfft2d_tiny(fft_size, freq, real, planes, h, w, pad_u, pad_l, bias, bias_period,
                                            static_cast<hipStream_t>(stream)), "irfft2d");
@@ -638,6 +691,32 @@ int fbfc_update_output_bias(float *output, const float *bias, int batch, int pla
     if (batch < 1 || planes < 1 || h < 1 || w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
     FBFC_TRY(fbfc::launch_bias_add(output, bias, batch, planes, h * w, static_cast<hipStream_t>(stream)),
              "bias add");
+    return FBFC_OK;
+}
+
+int fbfc_update_output_bias_strided(float *output, const float *bias, int batch, int planes, int h, int w,
+                                    long stride_b, long stride_f, long stride_h, long stride_w,
+                                    long bias_stride, void *stream)
+{
+    if (output == nullptr || bias == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (batch < 1 || planes < 1 || h < 1 || w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    FBFC_TRY(fbfc::launch_bias_add_strided(output, bias, batch, planes, h, w, stride_b, stride_f, stride_h,
+                                           stride_w, bias_stride, static_cast<hipStream_t>(stream)),
+             "bias add");
+    return FBFC_OK;
+}
+
+int fbfc_acc_grad_parameters_bias_strided(const float *grad_output, float *grad_bias, float scale, int batch,
+                                          int planes, int h, int w, long stride_b, long stride_f,
+                                          long stride_h, long stride_w, long bias_stride, float *scratch,
+                                          void *stream)
+{
+    if (grad_output == nullptr || grad_bias == nullptr || scratch == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (batch < 1 || planes < 1 || h < 1 || w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    FBFC_TRY(fbfc::launch_bias_grad_strided(grad_output, grad_bias, scale, batch, planes, h, w, stride_b,
+                                            stride_f, stride_h, stride_w, bias_stride, scratch,
+                                            static_cast<hipStream_t>(stream)), "bias grad");
     return FBFC_OK;
 }
 

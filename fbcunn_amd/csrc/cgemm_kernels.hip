@@ -15,7 +15,8 @@
 // block; tile 64 x 64 x 16 complex per step with register-prefetch double buffering through LDS.
 #include <hip/hip_runtime.h>
 
-#include <cstdlib>
+#include <atomic>
+#include <cstdio>
 
 #include "kernels.h"
 #include "store_nt.h"
@@ -636,17 +637,20 @@ static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_
     return hipGetLastError();
 }
 
-// FBFC_CGEMM_SPLITK forces a kernel variant (for measurements): 0 = register-staged LDS tiles,
-// 8 = LDS-direct tiles, 9 = hybrid of LDS-direct tiles and split blocks, 1 / 2 / 4 = register-fed
-// kernel with that many waves per block.
-static int splitk_override()
+// A forced kernel variant (for measurements; see fbfc_debug_force_contraction_kernel): -1 = the
+// shape rule below, 0 = register-staged LDS tiles, 8 = LDS-direct tiles, 9 = hybrid of LDS-direct
+// tiles and split blocks, 1 / 2 / 4 = register-fed kernel with that many waves per block.
+static std::atomic<int> g_force_variant{-1};
+void cgemm_force_variant(int v) { g_force_variant.store(v); }
+static int splitk_override() { return g_force_variant.load(std::memory_order_relaxed); }
+
+// name of the kernel the last contraction launched from this thread chose
+static thread_local char g_last_kernel[48] = "";
+const char *cgemm_last_kernel() { return g_last_kernel; }
+static void note_kernel(const char *base, int mode, int variant)
 {
-    static int v = -2;
-    if (v == -2) {
-        const char *e = getenv("FBFC_CGEMM_SPLITK");
-        v = (e != nullptr) ? atoi(e) : -1;
-    }
-    return v;
+    if (variant >= 0) snprintf(g_last_kernel, sizeof g_last_kernel, "%s<%d, %d>", base, mode, variant);
+    else snprintf(g_last_kernel, sizeof g_last_kernel, "%s<%d>", base, mode);
 }
 
 template <int MODE>
@@ -677,6 +681,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
             const int direct_wgs = q_direct * t64;
             const int split_tiles = q_split * (m / 32) * (n / 32);  // one workgroup per 32x32 block
             const int chunk_direct = (direct_wgs + 7) / 8, chunk_split = (split_tiles + 7) / 8;
+            note_kernel("cgemm_hybrid_kernel", MODE, -1);
             hipLaunchKernelGGL(cgemm_hybrid_kernel<MODE>, dim3((unsigned)((chunk_direct + chunk_split) * 8)),
                                dim3(256), 0, s, reinterpret_cast<const float2 *>(A),
                                reinterpret_cast<const float2 *>(B), reinterpret_cast<float2 *>(C), m, n, k,
@@ -693,6 +698,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
         const int t96 = n / 96;
         const long tot = (long)n_freq * tilesM * t96;
         const int ch = (int)((tot + 7) / 8);
+        note_kernel("cgemm_ldsdirect_kernel", MODE, 3);
         hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 3>), dim3((unsigned)(ch * 8)), dim3(384), 0, s,
                            reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                            reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, t96, (int)tot, ch,
@@ -707,18 +713,21 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
         else if (tot32 < 4 * 1024 && (k % 64) == 0) sk = 4;
         else if (tot32 < 8 * 1024 && (k % 32) == 0) sk = 2;
         else sk = 1;
+        if ((sk == 4 && (k % 64) == 0) || (sk == 2 && (k % 32) == 0) || sk == 1) note_kernel("cgemm_splitk_kernel", MODE, sk);
         if (sk == 4 && (k % 64) == 0) return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
         if (sk == 2 && (k % 32) == 0) return launch_splitk<MODE, 2>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
         if (sk == 1) return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
     }
     const int chunk = (int)((total + 7) / 8);
     if (direct_ok && force != 0) {
+        note_kernel("cgemm_ldsdirect_kernel", MODE, 2);
         hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 2>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                            reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                            reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
                            (int)total, chunk, fm);
         return hipGetLastError();
     }
+    note_kernel("cgemm_freq_kernel", MODE, -1);
     hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                        reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,

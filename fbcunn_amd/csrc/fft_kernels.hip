@@ -22,6 +22,8 @@
 // The inverse kernel is the mirror image and adds the bias while cropping.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "bias_dc.h"
 #include "fft_regs.h"
 #include "kernels.h"
@@ -382,8 +384,7 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
     constexpr int LDR = Canvas<N>::LDR;
     // Planes of odd height and width are staged raw, by asynchronous LDS-direct loads (their rows fall on
     // different LDS banks by themselves); windowed operands, even sizes (a 32 x 32 plane staged raw puts
-    // every row on the same banks) and N = 128 (one-plane rounds need not be 16-byte multiples) are staged
-    // as zero-padded canvas rows.
+    // every row on the same banks) and N = 128 are staged as zero-padded canvas rows.
     static_assert(!RAW || (!WIN && N <= 64), "raw staging: plain operands, N <= 64");
     const int zrow = S::TP * h;  // canvas staging: an all-zero row for canvas rows outside the plane
     // raw staging: bit x of colmask = canvas column x lies inside the plane
@@ -749,16 +750,17 @@ static long fwd_blocks(long planes)
     return blocks;
 }
 
-template <int N>
+template <int N, bool SMALL = false>
 static FwdJob make_job(const FwdArgs &a)
 {
-    using S = FftShape<N, false>;
+    using S = FftShape<N, false, SMALL>;
     FwdJob j;
     j.in = a.in;
     j.out = reinterpret_cast<float2 *>(a.out);
     j.planes = a.planes;
     j.h = a.h; j.w = a.w; j.padU = a.padU; j.padL = a.padL;
-    j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::T * a.h * a.w) % 4 == 0);
+    // every staging round starts TP planes after the previous one: all of them 16-byte aligned
+    j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
     j.tbl_off = 0;
     j.herm = a.herm;
     j.win = a.win;
@@ -780,23 +782,16 @@ static bool raw_ok(const FwdArgs &a) { return (a.h & 1) && (a.w & 1) && !a.win.o
 template <int N, bool WIN, int NZ, bool RAW>
 static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
 {
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rfft2d_kernel<N, WIN, NZ, RAW>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
     size_t lds = fft_lds_bytes<N, false, (NZ < N)>(a.h, a.w, a.padU);
     const long blocks0 = fwd_blocks<N>(a.planes);
     long blocks = blocks0;
-    FwdJob j0 = make_job<N>(a);
+    FwdJob j0 = make_job<N, (NZ < N)>(a);
     FwdJob j1 = j0;
     if (second != nullptr) {
         const size_t lds1 = fft_lds_bytes<N, false, (NZ < N)>(second->h, second->w, second->padU);
         if (lds1 > lds) lds = lds1;
         blocks += fwd_blocks<N>(second->planes);
-        j1 = make_job<N>(*second);
+        j1 = make_job<N, (NZ < N)>(*second);
     }
     if (WIN) {  // the window table sits behind the tile / staging area
         j0.tbl_off = j1.tbl_off = (int)(lds / sizeof(float));
@@ -821,19 +816,13 @@ template <int N, bool WIN, int PHASES>
 static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s)
 {
     using S = FftShape<N, true, false, PHASES>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&irfft2d_kernel<N, WIN, PHASES>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
     size_t lds = fft_lds_bytes<N, true, false, PHASES>(a.h, a.w, a.padU);
     const int tbl_off = (int)(lds / sizeof(float));
     if (WIN) lds += S::T * sizeof(int4);
     long blocks = (a.planes + S::T - 1) / S::T;
     if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
-    const int vec4 = ((reinterpret_cast<uintptr_t>(a.out) & 15) == 0) && (((long)S::T * a.h * a.w) % 4 == 0);
+    // every copy-out round starts TP planes after the previous one: all of them 16-byte aligned
+    const int vec4 = ((reinterpret_cast<uintptr_t>(a.out) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
     Window win = a.win;
     win.remap = window_remap_ok<S::T>(a.win, a.planes);
     const BiasGradJob bgrad = {reinterpret_cast<const float2 *>(a.go_freq), a.grad_bias, a.scale, a.batch,
@@ -859,7 +848,63 @@ static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
 }
 
 // the kernels address a frequency row with 32-bit lane offsets
-static bool planes_ok(int N, long planes) { return planes > 0 && (long)(N / 2 + 1) * planes * 8 < (1L << 31); }
+long fft_max_planes(int N) { return ((1L << 31) - 1) / ((long)(N / 2 + 1) * 8); }
+static bool planes_ok(int N, long planes) { return planes > 0 && planes <= fft_max_planes(N); }
+
+// Raises the dynamic-LDS limit of every kernel instantiation on the current device.  Called once per
+// device (plan creation, first stand-alone transform), so that no launch makes an attribute call:
+// launches may then be captured into a graph whatever shape comes first.
+template <class K>
+static hipError_t raise_lds_limit(K *kernel)
+{
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               160 * 1024);
+}
+
+template <int N>
+static hipError_t raise_lds_limits_windowed()
+{
+    hipError_t e = raise_lds_limit(&rfft2d_kernel<N, true, N, false>);
+    if (e == hipSuccess) e = raise_lds_limit(&irfft2d_kernel<N, true, 0>);
+    if (e == hipSuccess && N == 32) e = raise_lds_limit(&irfft2d_kernel<N, true, (N == 32 ? 2 : 0)>);
+    return e;
+}
+
+template <int N>
+static hipError_t raise_lds_limits_plain()
+{
+    hipError_t e = raise_lds_limit(&rfft2d_kernel<N, false, N, false>);
+    if constexpr (N <= 64) {
+        if (e == hipSuccess) e = raise_lds_limit(&rfft2d_kernel<N, false, N, true>);
+    }
+    if (e == hipSuccess) e = raise_lds_limit(&irfft2d_kernel<N, false, 0>);
+    if (e == hipSuccess && N == 32) e = raise_lds_limit(&irfft2d_kernel<N, false, (N == 32 ? 2 : 0)>);
+    return e;
+}
+
+hipError_t fft_prepare_device()
+{
+    static std::mutex mu;
+    static bool done[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (done[dev]) return hipSuccess;
+    e = raise_lds_limits_plain<8>();
+    if (e == hipSuccess) e = raise_lds_limits_plain<16>();
+    if (e == hipSuccess) e = raise_lds_limits_plain<32>();
+    if (e == hipSuccess) e = raise_lds_limits_plain<64>();
+    if (e == hipSuccess) e = raise_lds_limits_plain<128>();
+    if (e == hipSuccess) e = raise_lds_limit(&rfft2d_kernel<64, false, 16, false>);
+    if (e == hipSuccess) e = raise_lds_limit(&rfft2d_kernel<64, false, 16, true>);
+    if (e == hipSuccess) e = raise_lds_limits_windowed<8>();
+    if (e == hipSuccess) e = raise_lds_limits_windowed<16>();
+    if (e == hipSuccess) e = raise_lds_limits_windowed<32>();
+    if (e == hipSuccess) done[dev] = true;
+    return e;
+}
 
 static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s)
 {

@@ -57,6 +57,13 @@ struct InvArgs {
 };
 hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s);
 
+// Largest number of planes one launch of an N x N transform takes (the kernels address a frequency
+// row of the spectrum with 32-bit byte offsets): floor((2^31 - 1) / ((N/2 + 1) * 8)).
+long fft_max_planes(int N);
+// Raises the dynamic-LDS limit of every transform kernel on the current device, once per device.
+// After it no launch makes an attribute call (launches may be captured whatever shape comes first).
+hipError_t fft_prepare_device();
+
 // fft_small.hip ------------------------------------------------------------------
 // 1-D batched transforms, N in {2,4,...,128}: rows of n reals at pad_l of the N-point canvas
 // <-> (rows, N/2+1) complex, row-major; the inverse is unnormalised.
@@ -90,6 +97,13 @@ inline int hermitian_count(int N) { return (N / 2 + 1) * (N / 2 + 1) + (N / 2 - 
 hipError_t launch_cgemm_freq_map(int mode, const float *A, const float *B, float *C, int n_freq, FreqMap fm,
                                  int m, int n, int k, float alpha, int accumulate, hipStream_t s);
 
+// Name of the kernel the last contraction launched from the calling thread chose ("" before the first).
+const char *cgemm_last_kernel();
+// Measurement knob: -1 = choose by shape; 0 = register-staged LDS tiles, 8 = LDS-direct tiles,
+// 9 = hybrid of LDS-direct tiles and split blocks, 1 / 2 / 4 = register-fed kernel with that many
+// waves per block (falls back to the shape rule where the forced variant cannot run the shape).
+void cgemm_force_variant(int v);
+
 // bias_kernels.hip ---------------------------------------------------------------
 hipError_t launch_bias_add(float *out, const float *bias, int batch, int planes, int hw,
                            hipStream_t s);
@@ -97,6 +111,12 @@ size_t bias_grad_scratch_bytes(int batch, int planes);
 hipError_t launch_bias_grad(const float *grad_out, float *grad_bias, float scale, int batch,
                             int planes, int hw, float *scratch, hipStream_t s);
 
+// Strided forms: element (b, f, r, c) at b * sb + f * sf + r * sh + c * sw floats, bias[f] at f * bias_stride.
+hipError_t launch_bias_add_strided(float *out, const float *bias, int batch, int planes, int h, int w,
+                                   long sb, long sf, long sh, long sw, long bias_stride, hipStream_t s);
+hipError_t launch_bias_grad_strided(const float *grad_out, float *grad_bias, float scale, int batch,
+                                    int planes, int h, int w, long sb, long sf, long sh, long sw,
+                                    long bias_stride, float *scratch, hipStream_t s);
 // freq = frequency-major spectrum of grad_out (its first frequency row holds the plane sums)
 hipError_t launch_bias_grad_dc(const float *freq, float *grad_bias, float scale, int batch, int planes,
                                hipStream_t s);

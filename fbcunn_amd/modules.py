@@ -28,14 +28,14 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def _check_tensor(t, name, ndim=None):
+def _check_tensor(t, name, ndim=None, strided=False):
     if not isinstance(t, torch.Tensor) or not t.is_cuda:
         raise TypeError("%s: CUDA support only!" % name)   # the reference's assert message
     if t.dtype != torch.float32:
         raise TypeError("%s must be float32" % name)
     if ndim is not None and t.dim() != ndim:
         raise ValueError("%s must be %d-D" % (name, ndim))
-    if not t.is_contiguous():
+    if not strided and not t.is_contiguous():
         raise ValueError("%s must be contiguous" % name)
 
 
@@ -150,6 +150,13 @@ class SpatialConvolutionFFT:
         _check_tensor(input, "input", 4)
         if input.size(1) != self.nInputPlane:
             raise ValueError("input has %d planes, module expects %d" % (input.size(1), self.nInputPlane))
+
+    def contractionKernel(self, input):
+        """Name of the contraction kernel the last pass on this input shape launched."""
+        plan = self._plan_for(input.size(0), input.size(2), input.size(3))
+        buf = ctypes.create_string_buffer(64)
+        check(lib().fbfc_plan_contraction_kernel(plan.handle, buf, len(buf)))
+        return buf.value.decode()
 
     def stageTimes(self, input):
         """Mean ms per launch of each stage of the last pass run with self.timed = reps > 0 (dict)."""
@@ -360,21 +367,32 @@ def transposeMM(A, B, C, invNorm, conjugateTransposeA, conjugateTransposeB, accu
 
 
 def updateOutputBias(output, bias):
-    """updateOutputBiasFFI (src/ConvolutionBias.cu:256-260)."""
-    _check_tensor(output, "output", 4)
-    _check_tensor(bias, "bias", 1)
+    """updateOutputBiasFFI (src/ConvolutionBias.cu:256-260); like the reference's kernel it takes
+    non-contiguous tensors (test/BiasTest.cpp:38-63)."""
+    _check_tensor(output, "output", 4, strided=True)
+    _check_tensor(bias, "bias", 1, strided=True)
     B, F, h, w = output.shape
-    check(lib().fbfc_update_output_bias(_ptr(output), _ptr(bias), B, F, h, w, _stream()))
+    if output.is_contiguous() and bias.is_contiguous():
+        check(lib().fbfc_update_output_bias(_ptr(output), _ptr(bias), B, F, h, w, _stream()))
+    else:
+        check(lib().fbfc_update_output_bias_strided(_ptr(output), _ptr(bias), B, F, h, w, *output.stride(),
+                                                    bias.stride(0), _stream()))
     return output
 
 
 def accGradParametersBias(gradOutput, gradBias, scale=1.0):
-    """accGradParametersBiasFFI (src/ConvolutionBias.cu:262-274): gradBias is assigned."""
-    _check_tensor(gradOutput, "gradOutput", 4)
-    _check_tensor(gradBias, "gradBias", 1)
+    """accGradParametersBiasFFI (src/ConvolutionBias.cu:262-274): gradBias is assigned.  Takes
+    non-contiguous tensors (test/BiasTest.cpp:186-222)."""
+    _check_tensor(gradOutput, "gradOutput", 4, strided=True)
+    _check_tensor(gradBias, "gradBias", 1, strided=True)
     B, F, h, w = gradOutput.shape
     nbytes = lib().fbfc_bias_grad_scratch_bytes(B, F)
     scratch = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=gradOutput.device)
-    check(lib().fbfc_acc_grad_parameters_bias(_ptr(gradOutput), _ptr(gradBias), ctypes.c_float(scale),
-                                              B, F, h, w, _ptr(scratch), _stream()))
+    if gradOutput.is_contiguous() and gradBias.is_contiguous():
+        check(lib().fbfc_acc_grad_parameters_bias(_ptr(gradOutput), _ptr(gradBias), ctypes.c_float(scale),
+                                                  B, F, h, w, _ptr(scratch), _stream()))
+    else:
+        check(lib().fbfc_acc_grad_parameters_bias_strided(_ptr(gradOutput), _ptr(gradBias), ctypes.c_float(scale),
+                                                          B, F, h, w, *gradOutput.stride(), gradBias.stride(0),
+                                                          _ptr(scratch), _stream()))
     return gradBias

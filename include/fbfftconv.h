@@ -74,7 +74,10 @@ const char *fbfc_last_error(void);
  * choice do (stride 1: SpatialConvolutionFFT.lua:176, SpatialConvolutionFBFFT.lua:60-61;
  * pad < kernel: SpatialConvolutionFBFFT.lua:93-95; nextPowerOf2: SpatialConvolutionFFT.lua:875-882)
  * and fills *info.  FFT sizes above 128 are FBFC_ERR_UNSUPPORTED_SIZE (the reference's
- * fbfft stops at 128 as well); sizes below 8 run on an 8 x 8 canvas. */
+ * fbfft stops at 128 as well); sizes below 8 run on an 8 x 8 canvas.  A tensor of more than
+ * floor((2^31 - 1) / ((N/2 + 1) * 8)) planes (batch x planes, or output x input planes; 8.1 million
+ * at N = 64) is FBFC_ERR_UNSUPPORTED_SIZE too, with the count in the message: one launch addresses
+ * a frequency row of the spectrum with 32-bit offsets. */
 int fbfc_plan_query(const fbfc_conv_desc *desc, fbfc_plan_info *info);
 
 /* Plans -----------------------------------------------------------------------
@@ -154,6 +157,16 @@ enum { FBFC_STAGE_FFT_A = 0,   /* the forward-FFT launch: both operands of the p
 int fbfc_plan_set_timed(fbfc_plan *plan, int reps);
 /* Milliseconds of each stage of the last timed pass (0 for a stage not run). */
 int fbfc_plan_stage_ms(const fbfc_plan *plan, float *ms, int n);
+/* Name of the contraction kernel the plan's last pass launched (the library picks one of several
+ * by shape), as a profiler trace shows it, e.g. "cgemm_hybrid_kernel<0>"; "" before the first pass.
+ * The counterpart of the kernel names the reference's timed wrappers log
+ * (src/CuBLASWrapperLua.cpp:39-137). */
+int fbfc_plan_contraction_kernel(const fbfc_plan *plan, char *name, size_t n);
+/* Measurement knob (no counterpart in the reference): forces the contraction kernel variant for the
+ * whole process.  -1 = choose by shape (default); 0 = register-staged LDS tiles with bounds checks,
+ * 8 = LDS-direct tiles, 9 = LDS-direct tiles plus split blocks, 1 / 2 / 4 = register-fed kernel
+ * with that many waves per block.  A variant that cannot run a shape falls back to the shape rule. */
+int fbfc_debug_force_contraction_kernel(int variant);
 
 /* Stand-alone stages ------------------------------------------------------------
  * Replaces FFTWrapper_fft with fbfft (src/fft/FFTWrapperLua.cpp:209-272 ->
@@ -196,6 +209,14 @@ int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq,
 int fbfc_update_output_bias(float *output, const float *bias, int batch, int planes,
                             int h, int w, void *stream);
 
+/* The same on a non-contiguous feature-map tensor, which the reference's bias kernels accept
+ * (src/ConvolutionBias.cu:39-51 takes strided DeviceTensors; test/BiasTest.cpp:38-63 transposes two
+ * dimensions): element (b, f, r, c) lies at b*stride_b + f*stride_f + r*stride_h + c*stride_w floats
+ * from `output`, bias[f] at f*bias_stride floats from `bias`. */
+int fbfc_update_output_bias_strided(float *output, const float *bias, int batch, int planes,
+                                    int h, int w, long stride_b, long stride_f, long stride_h,
+                                    long stride_w, long bias_stride, void *stream);
+
 /* Replaces accGradParametersBiasFFI (src/ConvolutionBias.cu:262-274):
  * grad_bias[f] = scale * sum_{b,r,c} grad_output[b][f][r][c] (assignment).
  * scratch must hold fbfc_bias_grad_scratch_bytes(batch, planes) bytes. */
@@ -203,6 +224,12 @@ size_t fbfc_bias_grad_scratch_bytes(int batch, int planes);
 int fbfc_acc_grad_parameters_bias(const float *grad_output, float *grad_bias, float scale,
                                   int batch, int planes, int h, int w,
                                   float *scratch, void *stream);
+/* The same on a non-contiguous grad_output (src/ConvolutionBias.cu:61-97; test/BiasTest.cpp:186-222);
+ * strides in floats as for fbfc_update_output_bias_strided; scratch as above (dense). */
+int fbfc_acc_grad_parameters_bias_strided(const float *grad_output, float *grad_bias, float scale,
+                                          int batch, int planes, int h, int w, long stride_b,
+                                          long stride_f, long stride_h, long stride_w,
+                                          long bias_stride, float *scratch, void *stream);
 
 #ifdef __cplusplus
 }

@@ -70,6 +70,30 @@ def test_plan_rejections(kw, code, text):
     assert text in e.value.message
 
 
+def test_plan_refuses_more_planes_than_one_launch_addresses():
+    """One launch addresses a frequency row of the spectrum with 32-bit offsets: the limit is checked
+    when the plan is made and the message carries the numbers."""
+    n = 64
+    lim = (2 ** 31 - 1) // ((n // 2 + 1) * 8)
+    ok = _q(batch=lim // 4096, in_planes=4096, out_planes=16, in_h=55, in_w=55, k_h=9, k_w=9, pad_h=4, pad_w=4)
+    assert ok.fft_size == n
+    with pytest.raises(_lib.FbfcError) as e:
+        _q(batch=lim // 4096 + 1, in_planes=4096, out_planes=16, in_h=55, in_w=55, k_h=9, k_w=9, pad_h=4, pad_w=4)
+    assert e.value.code == _lib.ERR_UNSUPPORTED_SIZE
+    assert str(lim) in e.value.message and "input planes" in e.value.message
+    with pytest.raises(_lib.FbfcError) as e:
+        _q(batch=2, in_planes=8192, out_planes=8192, in_h=100, in_w=100, k_h=3, k_w=3, pad_h=1, pad_w=1)
+    assert e.value.code == _lib.ERR_UNSUPPORTED_SIZE and "output planes x input planes" in e.value.message
+    with pytest.raises(_lib.FbfcError) as e:    # tiles multiply the batch
+        _q(batch=4096, in_planes=512, out_planes=64, in_h=224, in_w=224, tile_h=16, tile_w=16)
+    assert e.value.code == _lib.ERR_UNSUPPORTED_SIZE and "batch x tiles" in e.value.message
+
+
+def test_debug_knob_validates_its_argument():
+    assert _lib.lib().fbfc_debug_force_contraction_kernel(3) == _lib.ERR_INVALID_ARGUMENT
+    assert _lib.lib().fbfc_debug_force_contraction_kernel(-1) == _lib.OK
+
+
 def test_scratch_size_query():
     assert _lib.lib().fbfc_bias_grad_scratch_bytes(128, 64) >= 64 * 4
     assert _lib.lib().fbfc_bias_grad_scratch_bytes(0, 64) == 0

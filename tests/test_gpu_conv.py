@@ -194,6 +194,59 @@ def test_acc_grad_overwrites_and_bias_functions(nn, oracle):
     np.testing.assert_allclose(host(out), oracle.bias_update_output(g, bias), rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("t1,t2", [(0, 1), (1, 3), (2, 3), (0, 2), (1, 1)])
+def test_bias_functions_take_non_contiguous_tensors(nn, oracle, t1, t2):
+    """test/BiasTest.cpp:38-63: the feature-map tensor is made with two dimensions swapped and
+    transposed back, so that it has the logical shape but an out-of-order memory layout."""
+    B, F, h, w = 5, 7, 6, 11
+    g = synth.uniform(56 + t1 + 4 * t2, (B, F, h, w))
+    sizes = [B, F, h, w]
+    sizes[t1], sizes[t2] = sizes[t2], sizes[t1]
+    store = torch.empty(sizes, device="cuda")
+    view = store.transpose(t1, t2)              # logical (B, F, h, w), non-contiguous unless t1 == t2
+    view.copy_(dev(g))
+    assert tuple(view.shape) == (B, F, h, w) and view.is_contiguous() == (t1 == t2)
+    gb_store = torch.full((F, 3), 123.0, device="cuda")
+    gb = gb_store[:, 1]                          # stride 3
+    nn.accGradParametersBias(view, gb, 0.25)
+    np.testing.assert_allclose(host(gb), oracle.bias_acc_grad_parameters(g, 0.25), rtol=5e-4, atol=1e-5)
+    assert (host(gb_store[:, 0]) == 123.0).all() and (host(gb_store[:, 2]) == 123.0).all()
+    bias = synth.uniform(77, (F,))
+    nn.updateOutputBias(view, dev(bias))
+    np.testing.assert_allclose(host(view.contiguous()), oracle.bias_update_output(g, bias), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("reuse", ["all", "output"])
+def test_second_acc_grad_under_reuse_transforms_its_own_grad_output(nn, oracle, reuse):
+    """updateOutput, accGradParameters, updateOutput, accGradParameters with another gradOutput and no
+    updateGradInput in between: the second accGradParameters must not take the spectrum of the first
+    gradOutput (memoryReuseOutput only covers the updateGradInput -> accGradParameters pair of one step,
+    fbcunn/SpatialConvolutionFBFFT.lua:305-322)."""
+    B, P, F, k, H, pad = 4, 6, 5, 3, 13, 1
+    x = synth.uniform(41, (B, P, H, H), stream=0)
+    w = synth.normal(41, (F, P, k, k), 0.0, 0.05, stream=1)
+    g1 = synth.uniform(41, (B, F, H, H), stream=3)
+    g2 = synth.uniform(42, (B, F, H, H), stream=3)
+    net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad, reuse)
+    net.weight.copy_(dev(w))
+    xd = dev(x)
+    p4 = (pad,) * 4
+    for g in (g1, g2, g1):
+        net.updateOutput(xd)
+        net.accGradParameters(xd, dev(g), 1.0)
+        _close(host(net.gradWeight), oracle.cross_correlation_reverse_valid(x, g, (1, 1), 1.0, p4), "gradWeight")
+        _close(host(net.gradBias), oracle.bias_acc_grad_parameters(g, 1.0), "gradBias")
+    # the pair the policy is for still shares the spectrum and gives the same numbers
+    net.updateOutput(xd)
+    net.updateGradInput(xd, dev(g2))
+    net.accGradParameters(xd, dev(g2), 1.0)
+    _close(host(net.gradWeight), oracle.cross_correlation_reverse_valid(x, g2, (1, 1), 1.0, p4), "gradWeight")
+    # two accGradParameters in a row with different gradOutput
+    net.accGradParameters(xd, dev(g1), 1.0)
+    _close(host(net.gradWeight), oracle.cross_correlation_reverse_valid(x, g1, (1, 1), 1.0, p4), "gradWeight")
+    net.cleanupBuffers()
+
+
 def test_module_argument_errors(nn):
     with pytest.raises(ValueError):
         nn.SpatialConvolutionFBFFT(3, 4, 3, 3, 2, 1)            # stride
