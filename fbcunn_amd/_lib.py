@@ -70,6 +70,7 @@ SIGNATURES = {
     "fbfc_acc_grad_parameters_bias_strided": (_i, [_vp, _vp, _f, _i, _i, _i, _i, _l, _l, _l, _l, _l, _vp, _vp]),
     "fbfc_bias_grad_scratch_bytes": (ctypes.c_size_t, [_i, _i]),
     "fbfc_acc_grad_parameters_bias": (_i, [_vp, _vp, _f, _i, _i, _i, _i, _vp, _vp]),
+    "fbfc_acc_grad_parameters_bias_noalloc": (_i, [_vp, _vp, _f, _i, _i, _i, _i, _vp]),
 }
 
 _lib = None

@@ -346,6 +346,7 @@ static int plan_create(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_
     set_geometry(p, tile_h, tile_w);
     hipError_t e = hipGetDevice(&p->device);
     if (e == hipSuccess) e = fbfc::fft_prepare_device();
+    if (e == hipSuccess) e = fbfc::bias_grad_noalloc_prepare();
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->in_freq), info.input_freq_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->w_freq), info.weight_freq_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->out_freq), info.output_freq_bytes);
@@ -734,6 +735,23 @@ int fbfc_acc_grad_parameters_bias(const float *grad_output, float *grad_bias, fl
     if (batch < 1 || planes < 1 || h < 1 || w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
     FBFC_TRY(fbfc::launch_bias_grad(grad_output, grad_bias, scale, batch, planes, h * w, scratch,
                                     static_cast<hipStream_t>(stream)), "bias grad");
+    return FBFC_OK;
+}
+
+int fbfc_acc_grad_parameters_bias_noalloc(const float *grad_output, float *grad_bias, float scale,
+                                          int batch, int planes, int h, int w, void *stream)
+{
+    if (grad_output == nullptr || grad_bias == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (batch < 1 || planes < 1 || h < 1 || w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    if (planes > fbfc::bias_grad_noalloc_max_planes()) {
+        char buf[160];
+        std::snprintf(buf, sizeof buf,
+                      "%d planes exceed the %d the fixed workspace holds; use fbfc_acc_grad_parameters_bias "
+                      "with a workspace of your own", planes, fbfc::bias_grad_noalloc_max_planes());
+        return fail(FBFC_ERR_UNSUPPORTED_SIZE, buf);
+    }
+    FBFC_TRY(fbfc::launch_bias_grad_noalloc(grad_output, grad_bias, scale, batch, planes, h * w,
+                                            static_cast<hipStream_t>(stream)), "bias grad (fixed workspace)");
     return FBFC_OK;
 }
 

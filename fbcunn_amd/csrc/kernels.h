@@ -117,6 +117,14 @@ hipError_t launch_bias_add_strided(float *out, const float *bias, int batch, int
 hipError_t launch_bias_grad_strided(const float *grad_out, float *grad_bias, float scale, int batch,
                                     int planes, int h, int w, long sb, long sf, long sh, long sw,
                                     long bias_stride, float *scratch, hipStream_t s);
+// bias_noalloc.hip: the bias gradient with its partial sums in a fixed device array (no allocation,
+// no workspace argument); at most bias_grad_noalloc_max_planes() planes.  prepare() looks the array
+// up on the current device (the first launch does so too).
+int bias_grad_noalloc_max_planes();
+hipError_t bias_grad_noalloc_prepare();
+hipError_t launch_bias_grad_noalloc(const float *grad_out, float *grad_bias, float scale, int batch,
+                                    int planes, int hw, hipStream_t s);
+
 // freq = frequency-major spectrum of grad_out (its first frequency row holds the plane sums)
 hipError_t launch_bias_grad_dc(const float *freq, float *grad_bias, float scale, int batch, int planes,
                                hipStream_t s);

@@ -231,6 +231,17 @@ int fbfc_acc_grad_parameters_bias_strided(const float *grad_output, float *grad_
                                           long stride_f, long stride_h, long stride_w,
                                           long bias_stride, float *scratch, void *stream);
 
+/* fbfc_acc_grad_parameters_bias without the workspace argument, for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  The partial sums live in a fixed 256 KB
+ * array in device memory that every GPU the library runs on holds until the process ends; the call
+ * allocates and frees nothing.  At most 4096 planes (FBFC_ERR_UNSUPPORTED_SIZE beyond, with the
+ * limit in the message).  Results equal those of fbfc_acc_grad_parameters_bias bit for bit.  All
+ * calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
+ * threads) race and must be serialised by the caller. */
+int fbfc_acc_grad_parameters_bias_noalloc(const float *grad_output, float *grad_bias, float scale,
+                                          int batch, int planes, int h, int w, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
