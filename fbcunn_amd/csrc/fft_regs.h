@@ -1,8 +1,9 @@
 // In-register complex FFT of a compile-time power-of-two length.
 //
 // One lane holds a whole length-N complex sequence in registers (re[N], im[N])
-// and transforms it with fully unrolled radix-2 decimation-in-frequency
-// butterflies.  Every array index and every twiddle factor is a compile-time
+// and transforms it with fully unrolled radix-2 butterflies (input in natural order,
+// one twiddle per block applied before the add/subtract, so that a butterfly is six
+// multiply-adds).  Every array index and every twiddle factor is a compile-time
 // constant, so the arrays never leave the register file.  The result is left in
 // bit-reversed order: X[k] is found at position fbfc::brev<N>(k).
 #pragma once
@@ -65,74 +66,71 @@ __host__ __device__ __forceinline__ void static_for(F &&f) {
 }
 
 // ---- butterflies ----------------------------------------------------------------
-// One DIF butterfly of a length-LEN sub-transform starting at OFF:
-//   a' = a + b ;  b' = (a - b) * W,  W = exp(-/+ 2 pi i K / LEN)  (- forward, + inverse)
-template <int LEN, int OFF, int K, bool INV>
-__host__ __device__ __forceinline__ void butterfly(float *re, float *im) {
-    constexpr int H = LEN / 2;
-    const float ar = re[OFF + K], ai = im[OFF + K];
-    const float br = re[OFF + K + H], bi = im[OFF + K + H];
-    re[OFF + K] = ar + br;
-    im[OFF + K] = ai + bi;
-    const float dr = ar - br, di = ai - bi;
-    if constexpr (K == 0) {
-        re[OFF + K + H] = dr;
-        im[OFF + K + H] = di;
-    } else if constexpr (4 * K == LEN) {  // W = -i (forward) / +i (inverse)
-        re[OFF + K + H] = INV ? -di : di;
-        im[OFF + K + H] = INV ? dr : -dr;
-    } else if constexpr (8 * K == LEN) {  // W = (1 -/+ i) / sqrt2
-        constexpr float s = 0.70710678118654752440f;
-        re[OFF + K + H] = INV ? (dr - di) * s : (dr + di) * s;
-        im[OFF + K + H] = INV ? (dr + di) * s : (di - dr) * s;
-    } else if constexpr (8 * K == 3 * LEN) {  // W = (-1 -/+ i) / sqrt2
-        constexpr float s = 0.70710678118654752440f;
-        re[OFF + K + H] = INV ? (-dr - di) * s : (di - dr) * s;
-        im[OFF + K + H] = INV ? (dr - di) * s : (-dr - di) * s;
+// The transform of a block x[0..LEN) at register offset OFF is the "twisted" DFT
+//   X[k] = sum_n x[n] exp(-/+ 2 pi i n (k + theta) / LEN),   theta = TNUM / TDEN
+// (- forward, + inverse; theta = 0 for the whole sequence).  Splitting k = 2 k' + b gives
+//   y_b[n] = x[n] + (-1)^b T x[n + LEN/2],  T = exp(-/+ pi i theta),   n < LEN/2
+//   X[2 k' + b] = twisted DFT of y_b with theta' = (b + theta) / 2:
+// input in natural order, X[k] left at position brev(k), and ONE twiddle per block that multiplies
+// the second operand BEFORE the add/subtract.  That form fuses into multiply-adds:
+//   lo' = lo + T hi   (2 fma per component),   hi' = lo - T hi = 2 lo - lo'   (1 fma per component)
+// 6 instructions for a butterfly with a non-trivial twiddle (a decimation-in-frequency butterfly,
+// which multiplies after the subtraction, takes 8), 4 for T in {1, -/+ i}.
+template <int TNUM, int TDEN, bool INV>
+__host__ __device__ __forceinline__ void butterfly(float &ar, float &ai, float &br, float &bi) {
+    if constexpr (TNUM == 0) {  // T = 1
+        const float lr = ar + br, li = ai + bi;
+        br = ar - br;
+        bi = ai - bi;
+        ar = lr;
+        ai = li;
+    } else if constexpr (2 * TNUM == TDEN) {  // T = -i (forward) / +i (inverse): T b = (bi, -br) / (-bi, br)
+        const float pr = INV ? ar - bi : ar + bi, pi_ = INV ? ai + br : ai - br;
+        const float qr = INV ? ar + bi : ar - bi, qi = INV ? ai - br : ai + br;
+        ar = pr; ai = pi_;
+        br = qr; bi = qi;
     } else {
-        constexpr float wr = (float)cos2pi(K, LEN);
-        constexpr float wi = (float)(INV ? sin2pi(K, LEN) : -sin2pi(K, LEN));
-        re[OFF + K + H] = dr * wr - di * wi;
-        im[OFF + K + H] = dr * wi + di * wr;
+        constexpr float tr = (float)cos2pi(TNUM, 2 * TDEN);
+        constexpr float ti = (float)(INV ? sin2pi(TNUM, 2 * TDEN) : -sin2pi(TNUM, 2 * TDEN));
+        // lo' = a + T b
+        const float lr = __builtin_fmaf(tr, br, __builtin_fmaf(-ti, bi, ar));
+        const float li = __builtin_fmaf(tr, bi, __builtin_fmaf(ti, br, ai));
+        br = __builtin_fmaf(2.0f, ar, -lr);
+        bi = __builtin_fmaf(2.0f, ai, -li);
+        ar = lr;
+        ai = li;
     }
 }
 
-template <int LEN, int OFF, bool INV>
-__host__ __device__ __forceinline__ void fft_dif(float *re, float *im) {
+template <int LEN, int OFF, int TNUM, int TDEN, bool INV>
+__host__ __device__ __forceinline__ void fft_block(float *re, float *im) {
     if constexpr (LEN >= 2) {
-        static_for<LEN / 2>([&](auto k) { butterfly<LEN, OFF, decltype(k)::value, INV>(re, im); });
-        fft_dif<LEN / 2, OFF, INV>(re, im);
-        fft_dif<LEN / 2, OFF + LEN / 2, INV>(re, im);
+        constexpr int H = LEN / 2;
+        static_for<H>([&](auto kk) {
+            constexpr int k = decltype(kk)::value;
+            butterfly<TNUM, TDEN, INV>(re[OFF + k], im[OFF + k], re[OFF + k + H], im[OFF + k + H]);
+        });
+        fft_block<H, OFF, TNUM, 2 * TDEN, INV>(re, im);
+        fft_block<H, OFF + H, TDEN + TNUM, 2 * TDEN, INV>(re, im);
     }
 }
 
-// Input-pruned variant: only the first NZ inputs of the length-LEN sequence at OFF are non-zero (the
-// caller leaves literal zeros in the others).  While half the length is at least NZ a butterfly has
-// b = 0, so a' = a and b' = a * W for the NZ leading positions and nothing at all for the others;
-// both halves then again have NZ leading non-zeros.
-template <int LEN, int OFF, int K, bool INV>
-__host__ __device__ __forceinline__ void butterfly_b0(float *re, float *im) {
-    constexpr int H = LEN / 2;
-    const float ar = re[OFF + K], ai = im[OFF + K];
-    if constexpr (K == 0) {
-        re[OFF + H] = ar;
-        im[OFF + H] = ai;
-    } else {
-        constexpr float wr = (float)cos2pi(K, LEN);
-        constexpr float wi = (float)(INV ? sin2pi(K, LEN) : -sin2pi(K, LEN));
-        re[OFF + K + H] = ar * wr - ai * wi;
-        im[OFF + K + H] = ar * wi + ai * wr;
-    }
-}
-
-template <int LEN, int OFF, bool INV, int NZ>
-__host__ __device__ __forceinline__ void fft_dif_nz(float *re, float *im) {
+// Input-pruned variant: only the first NZ inputs of the block are non-zero (the caller leaves
+// literal zeros in the others).  While half the block length is at least NZ every butterfly has
+// hi = 0, so lo' = hi' = lo: the second half is a copy of the first, whatever the twiddle.
+template <int LEN, int OFF, int TNUM, int TDEN, bool INV, int NZ>
+__host__ __device__ __forceinline__ void fft_block_nz(float *re, float *im) {
     if constexpr (LEN / 2 >= NZ && LEN >= 2) {
-        static_for<NZ>([&](auto k) { butterfly_b0<LEN, OFF, decltype(k)::value, INV>(re, im); });
-        fft_dif_nz<LEN / 2, OFF, INV, NZ>(re, im);
-        fft_dif_nz<LEN / 2, OFF + LEN / 2, INV, NZ>(re, im);
+        constexpr int H = LEN / 2;
+        static_for<NZ>([&](auto kk) {
+            constexpr int k = decltype(kk)::value;
+            re[OFF + k + H] = re[OFF + k];
+            im[OFF + k + H] = im[OFF + k];
+        });
+        fft_block_nz<H, OFF, TNUM, 2 * TDEN, INV, NZ>(re, im);
+        fft_block_nz<H, OFF + H, TDEN + TNUM, 2 * TDEN, INV, NZ>(re, im);
     } else {
-        fft_dif<LEN, OFF, INV>(re, im);
+        fft_block<LEN, OFF, TNUM, TDEN, INV>(re, im);
     }
 }
 
@@ -140,13 +138,13 @@ __host__ __device__ __forceinline__ void fft_dif_nz(float *re, float *im) {
 template <int N, int NZ, bool INV>
 __host__ __device__ __forceinline__ void fft_inplace_nz(float (&re)[N], float (&im)[N]) {
     static_assert(NZ >= 1 && NZ <= N, "NZ leading non-zero inputs");
-    fft_dif_nz<N, 0, INV, NZ>(re, im);
+    fft_block_nz<N, 0, 0, 1, INV, NZ>(re, im);
 }
 
 // Unnormalised length-N transform in place; output index k lives at brev<N>(k).
 template <int N, bool INV>
 __host__ __device__ __forceinline__ void fft_inplace(float (&re)[N], float (&im)[N]) {
-    fft_dif<N, 0, INV>(re, im);
+    fft_block<N, 0, 0, 1, INV>(re, im);
 }
 
 }  // namespace fbfc
