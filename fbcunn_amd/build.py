@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libfbfftconv.so")
-SOURCES = ["api.cpp", "fft_kernels.hip", "fft_small.hip", "cgemm_kernels.hip", "bias_kernels.hip", "bias_noalloc.hip"]
+SOURCES = ["api.cpp", "fft_kernels.hip", "fft_large.hip", "fft_small.hip", "cgemm_kernels.hip", "bias_kernels.hip", "bias_noalloc.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
@@ -22,9 +22,15 @@ FLAGS = [
 ]
 
 
+# Per-file flags.  fft_large.hip: with common-code sinking the two role branches of the inverse kernel
+# end in one store through a pointer that selects between two register arrays, which forces both
+# into scratch memory.
+EXTRA_FLAGS = {"fft_large.hip": ["-mllvm", "-simplifycfg-sink-common=false"]}
+
+
 def _compile(src, report):
     out = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", out]
+    cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", out]
     if report:
         cmd.append("-Rpass-analysis=kernel-resource-usage")
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -35,7 +41,7 @@ def _compile(src, report):
 
 def build(report=False):
     os.makedirs(OBJ, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=6) as ex:
         results = list(ex.map(lambda s: _compile(s, report), SOURCES))
     objs = [o for o, _ in results]
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs

@@ -26,6 +26,7 @@
 
 #include "bias_dc.h"
 #include "fft_regs.h"
+#include "fft_stage.h"
 #include "kernels.h"
 #include "store_nt.h"
 
@@ -65,6 +66,12 @@ struct FftShape {
     static constexpr int LPR = THREADS / PH;
 };
 
+template <int N>
+__device__ __forceinline__ void store_freq(float2 *p, const float2 &v)
+{
+    store_freq_run<(FftShape<N, false>::T * 8 >= 128)>(p, v);
+}
+
 // Windowed operands: virtual plane v = (b * nt + tile) * d1 + c, so the workgroups of one tile (d1 / T of
 // them) are followed by those of the next tile -- on other XCDs, although neighbouring windows of one
 // image plane share cache lines (a 128-byte window row at an arbitrary offset touches two lines).  With
@@ -87,163 +94,6 @@ static int window_remap_ok(const Window &w, long planes)
     if (!w.on || w.d1 % T != 0) return 0;
     const long groups = planes / ((long)w.nt * w.d1) * (w.d1 / T);
     return groups % 8 == 0 && planes / T < (1L << 31);
-}
-
-// LDS staging area in canvas-row layout.  Row (p*h + r) of the staged planes starts at
-// (p*h + r) * LDR floats and holds the N canvas columns of that row: input column x sits
-// at padL + x, the margins are zero.  LDR = N + 4 floats keeps rows 16-byte aligned (the
-// row pass reads and writes them with 16-byte LDS accesses) while rotating them over the
-// banks.  The global side is the contiguous chunk of nrows * w floats.
-template <int N>
-struct Canvas {
-    static constexpr int LDR = N + 4;
-};
-
-// Workgroup -> plane-group mapping.  Workgroups are handed to the 8 XCDs round-robin.  When a
-// group's run per frequency is only half a 128-byte line (T*8 = 64 bytes), the two groups that
-// share each line are given to workgroups b and b+8: same XCD, dispatched back to back, so the
-// two halves meet in that XCD's L2 (one line fetched once / written back whole).
-template <int T>
-__device__ __forceinline__ long plane_group(unsigned bid)
-{
-    if constexpr (T * 8 >= 128) {
-        return (long)bid;
-    } else {
-        const unsigned cyc = bid >> 4, r = bid & 15u;
-        return (long)(2u * (cyc * 8u + (r & 7u)) + (r >> 3));
-    }
-}
-
-template <int N, bool TO_LDS, int NT = 256>
-__device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, int w, int padL,
-                                            int vec4, int tid)
-{
-    constexpr int LDR = Canvas<N>::LDR;
-    const int total = nrows * w;
-    int done = 0;
-    if (vec4) {
-        const int n4 = total >> 2;
-        float4 *g4 = reinterpret_cast<float4 *>(g);
-        int row = (tid * 4) / w, x = tid * 4 - row * w;
-        const int drow = (4 * NT) / w, dx = 4 * NT - drow * w;
-        if constexpr (TO_LDS) {
-            // U loads in flight per lane before the first one is waited for: one load per round trip
-            // would leave the memory system idle for most of the copy
-            constexpr int U = (N >= 64) ? 12 : 8;
-            for (int i0 = tid; i0 < n4; i0 += NT * U) {
-                float4 q[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int i = i0 + NT * u;
-                    if (i < n4) {
-                        if constexpr (N >= 64) {
-                            // planes of this size add up to tensors no cache holds until their next use:
-                            // stream them (measured at 16384 planes of 55 x 55: 160 -> 136 us; smaller
-                            // sizes got slower)
-                            const floatx4_nt t = __builtin_nontemporal_load(reinterpret_cast<const floatx4_nt *>(g4 + i));
-                            q[u] = make_float4(t.x, t.y, t.z, t.w);
-                        } else {
-                            q[u] = g4[i];
-                        }
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int i = i0 + NT * u;
-                    if (i < n4) {
-                        const float v[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
-                        int r_ = row, x_ = x;
-#pragma unroll
-                        for (int c = 0; c < 4; ++c) {
-                            smem[r_ * LDR + padL + x_] = v[c];
-                            if (++x_ == w) { x_ = 0; ++r_; }
-                        }
-                    }
-                    row += drow;
-                    x += dx;
-                    if (x >= w) { x -= w; ++row; }
-                }
-            }
-        } else {
-            for (int i = tid; i < n4; i += NT) {
-                float v[4];
-                int r_ = row, x_ = x;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    v[c] = smem[r_ * LDR + padL + x_];
-                    if (++x_ == w) { x_ = 0; ++r_; }
-                }
-                store_nt(g4 + i, make_float4(v[0], v[1], v[2], v[3]));
-                row += drow;
-                x += dx;
-                if (x >= w) { x -= w; ++row; }
-            }
-        }
-        done = n4 << 2;
-    }
-    {
-        const int first = done + tid;
-        int row = first / w, x = first - row * w;
-        const int drow = NT / w, dx = NT - drow * w;
-        for (int i = first; i < total; i += NT) {
-            float *sp = smem + row * LDR + padL + x;
-            if (TO_LDS) *sp = g[i]; else g[i] = *sp;
-            row += drow;
-            x += dx;
-            if (x >= w) { x -= w; ++row; }
-        }
-    }
-}
-
-// Spectrum stores.  Runs of whole 128-byte lines (N <= 32) are streamed past the cache (measured: 8.3 ->
-// 6.9 us for the 16384-plane N = 16 transform); the half-line runs of N >= 64 rely on the L2 to join the
-// two workgroups that share a line and stay ordinary stores.
-template <int N>
-__device__ __forceinline__ void store_freq(float2 *p, const float2 &v)
-{
-    if constexpr (FftShape<N, false>::T * 8 >= 128) store_nt(p, v);
-    else *p = v;
-}
-
-// Raw staging for the forward transform: the chunk of nfloats contiguous floats at g goes to LDS as it
-// lies, by LDS-direct loads (global_load_lds): no staging registers, no LDS store instructions and no
-// index arithmetic; the row pass then reads its rows at their (unaligned) places and masks the padding.
-// 16-byte pieces where the chunk allows (aligned16), 4-byte pieces for the rest.  The destination of a
-// wave instruction is wave-uniform; lane l lands at + l * size.  AUX: cache policy bits (2 = non-temporal).
-template <int AUX, int NT = 256>
-__device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloats, bool aligned16, int tid)
-{
-    const int wave = tid >> 6, lane = tid & 63;
-    int done = 0;
-    if (aligned16) {
-        const int n16 = nfloats >> 2;
-        for (int p0 = wave * 64; p0 < n16; p0 += NT) {
-            if (p0 + lane < n16)
-                __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1))) *)(g + 4 * (p0 + lane)),
-                    (void __attribute__((address_space(3))) *)(raw + 4 * p0), 16, 0, AUX);
-        }
-        done = n16 << 2;
-    }
-    for (int e0 = done + wave * 64; e0 < nfloats; e0 += NT) {
-        if (e0 + lane < nfloats)
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(g + e0 + lane),
-                                             (void __attribute__((address_space(3))) *)(raw + e0), 4, 0, AUX);
-    }
-}
-
-// Zeroes the margins of nrows canvas rows and the all-zero row kept at index zrow.
-template <int N, int NT = 256>
-__device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int w, int padL, int zrow,
-                                                    int tid)
-{
-    constexpr int LDR = Canvas<N>::LDR;
-    for (int row = tid; row < nrows; row += NT) {
-        float *sp = smem + row * LDR;
-        for (int c = 0; c < padL; ++c) sp[c] = 0.0f;
-        for (int c = padL + w; c < N; ++c) sp[c] = 0.0f;
-    }
-    if (tid < N) smem[zrow * LDR + tid] = 0.0f;
 }
 
 // ---------------------------------------------------------------------------------
@@ -323,18 +173,6 @@ __device__ __forceinline__ void copy_windows(float *smem, float *g, const int4 *
 // ---------------------------------------------------------------------------------
 // forward: real (planes,h,w) -> freq [N*(N/2+1)][planes] complex
 // ---------------------------------------------------------------------------------
-// One launch can transform two tensors of the same FFT size (the two forward FFTs of a pass):
-// workgroups [0, blocks0) work on job 0, the rest on job 1.
-struct FwdJob {
-    const float *in;
-    float2 *out;
-    long planes;
-    int h, w, padU, padL, vec4;
-    int tbl_off;  // windowed operand: float offset of the window table in LDS
-    int herm;     // leave out the entries (ky > N/2, kx in {0, N/2}): conjugates of (N - ky, kx)
-    Window win;
-};
-
 // NZ < N: planes of at most NZ x NZ at the canvas origin (convolution kernels): the transforms skip
 // the inputs that are known to be zero.
 template <int N, bool WIN, int NZ, bool RAW>
@@ -895,16 +733,19 @@ hipError_t fft_prepare_device()
     e = raise_lds_limits_plain<8>();
     if (e == hipSuccess) e = raise_lds_limits_plain<16>();
     if (e == hipSuccess) e = raise_lds_limits_plain<32>();
-    if (e == hipSuccess) e = raise_lds_limits_plain<64>();
-    if (e == hipSuccess) e = raise_lds_limits_plain<128>();
-    if (e == hipSuccess) e = raise_lds_limit(&rfft2d_kernel<64, false, 16, false>);
-    if (e == hipSuccess) e = raise_lds_limit(&rfft2d_kernel<64, false, 16, true>);
+    if (e == hipSuccess) e = fft_large_prepare_device();
+    if (e == hipSuccess) e = raise_lds_limit(&irfft2d_kernel<64, false, 0>);
+    if (e == hipSuccess) e = raise_lds_limit(&rfft2d_kernel<64, false, 64, false>);
+    if (e == hipSuccess) e = raise_lds_limit(&rfft2d_kernel<64, false, 64, true>);
     if (e == hipSuccess) e = raise_lds_limits_windowed<8>();
     if (e == hipSuccess) e = raise_lds_limits_windowed<16>();
     if (e == hipSuccess) e = raise_lds_limits_windowed<32>();
     if (e == hipSuccess) done[dev] = true;
     return e;
 }
+
+// N = 64: launches of at most this many planes take the 8-plane kernels of fft_large.hip
+constexpr long kSmallLaunch64 = 8192;
 
 static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s)
 {
@@ -919,22 +760,27 @@ static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStr
             default: return hipErrorInvalidValue;
         }
     }
-    if (N == 64) {
-        // planes of at most 16 x 16 at the origin (convolution kernels) take the variant that skips
-        // the zero inputs; a pair that holds such an operand is issued as two launches
-        auto small = [](const FwdArgs &x) { return x.h <= 16 && x.w <= 16 && x.padU == 0 && x.padL == 0; };
-        if (b != nullptr && (small(a) || small(*b))) {
-            const hipError_t e = dispatch_fwd(N, a, nullptr, s);
-            return e != hipSuccess ? e : dispatch_fwd(N, *b, nullptr, s);
-        }
-        if (b == nullptr && small(a)) return launch_fwd<64, false, 16>(a, nullptr, s);
-    }
     switch (N) {
         case 8: return launch_fwd<8, false>(a, b, s);
         case 16: return launch_fwd<16, false>(a, b, s);
         case 32: return launch_fwd<32, false>(a, b, s);
-        case 64: return launch_fwd<64, false>(a, b, s);
-        case 128: return launch_fwd<128, false>(a, b, s);
+        case 64: {
+            // planes of at most 16 x 16 at the origin (convolution kernels) take the variant that
+            // skips the zero inputs; a pair that holds such an operand is issued as two launches
+            auto small = [](const FwdArgs &x) { return x.h <= 16 && x.w <= 16 && x.padU == 0 && x.padL == 0; };
+            if (b != nullptr && (small(a) || small(*b))) {
+                const hipError_t e = dispatch_fwd(N, a, nullptr, s);
+                return e != hipSuccess ? e : dispatch_fwd(N, *b, nullptr, s);
+            }
+            // Launches of up to two rounds of 16-plane workgroups take the 8-plane kernel of
+            // fft_large.hip, two workgroups per CU: what it loses on its half-line runs it more than
+            // gains on balance (6144 planes of 55 x 55: 43.7 against 46.2 us); larger launches are
+            // faster with whole-line runs (16384 planes of 47 x 47: 107 against 112 us).
+            const long total = a.planes + (b != nullptr ? b->planes : 0);
+            if (small(a) || total <= kSmallLaunch64) return launch_rfft2d_large(N, a, b, s);
+            return launch_fwd<64, false>(a, b, s);
+        }
+        case 128: return launch_rfft2d_large(N, a, b, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -968,8 +814,8 @@ hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s)
         case 8: return launch_inv<8, false>(a, s);
         case 16: return launch_inv<16, false>(a, s);
         case 32: return launch_inv<32, false>(a, s);
-        case 64: return launch_inv<64, false>(a, s);
-        case 128: return launch_inv<128, false>(a, s);
+        case 64: return a.planes <= kSmallLaunch64 ? launch_irfft2d_large(N, a, s) : launch_inv<64, false>(a, s);
+        case 128: return launch_irfft2d_large(N, a, s);
         default: return hipErrorInvalidValue;
     }
 }

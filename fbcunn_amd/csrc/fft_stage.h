@@ -1,0 +1,191 @@
+// Pieces shared by the 2-D transform kernels: the LDS staging of real planes (canvas rows or the raw
+// chunk), the workgroup -> plane-group mapping and the spectrum stores.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+#include "store_nt.h"
+
+namespace fbfc {
+
+// LDS staging area in canvas-row layout.  Row (p*h + r) of the staged planes starts at
+// (p*h + r) * LDR floats and holds the N canvas columns of that row: input column x sits
+// at padL + x, the margins are zero.  LDR = N + 4 floats keeps rows 16-byte aligned (the
+// row pass reads and writes them with 16-byte LDS accesses) while rotating them over the
+// banks.  The global side is the contiguous chunk of nrows * w floats.
+template <int N>
+struct Canvas {
+    static constexpr int LDR = N + 4;
+};
+
+// Workgroup -> plane-group mapping.  Workgroups are handed to the 8 XCDs round-robin.  When a
+// group's run per frequency is only part of a 128-byte line (T*8 = 64 or 32 bytes), the G = 16 / T
+// groups that share each line are given to workgroups b, b+8, ... b+8(G-1): same XCD, dispatched back
+// to back, so the parts meet in that XCD's L2 (one line fetched once / written back whole).
+// GROUPS_PER_LINE < 0: derived from T.
+template <int T, int GROUPS_PER_LINE = -1>
+__device__ __forceinline__ long plane_group(unsigned bid)
+{
+    constexpr int G = GROUPS_PER_LINE > 0 ? GROUPS_PER_LINE : (T * 8 >= 128 ? 1 : 2);
+    if constexpr (G == 1) {
+        return (long)bid;
+    } else {
+        const unsigned cyc = bid / (8u * G), r = bid % (8u * G);
+        return (long)((unsigned)G * (cyc * 8u + (r & 7u)) + (r >> 3));
+    }
+}
+// the launch must cover whole cycles of that mapping
+template <int T, int GROUPS_PER_LINE = -1>
+inline long plane_group_blocks(long planes)
+{
+    constexpr int G = GROUPS_PER_LINE > 0 ? GROUPS_PER_LINE : (T * 8 >= 128 ? 1 : 2);
+    long blocks = (planes + T - 1) / T;
+    if (G > 1) blocks = (blocks + 8 * G - 1) / (8 * G) * (8 * G);
+    return blocks;
+}
+
+template <int N, bool TO_LDS, int NT = 256>
+__device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, int w, int padL,
+                                            int vec4, int tid)
+{
+    constexpr int LDR = Canvas<N>::LDR;
+    const int total = nrows * w;
+    int done = 0;
+    if (vec4) {
+        const int n4 = total >> 2;
+        float4 *g4 = reinterpret_cast<float4 *>(g);
+        int row = (tid * 4) / w, x = tid * 4 - row * w;
+        const int drow = (4 * NT) / w, dx = 4 * NT - drow * w;
+        if constexpr (TO_LDS) {
+            // U loads in flight per lane before the first one is waited for: one load per round trip
+            // would leave the memory system idle for most of the copy
+            constexpr int U = (N >= 64) ? 12 : 8;
+            for (int i0 = tid; i0 < n4; i0 += NT * U) {
+                float4 q[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int i = i0 + NT * u;
+                    if (i < n4) {
+                        if constexpr (N >= 64) {
+                            // planes of this size add up to tensors no cache holds until their next use:
+                            // stream them (measured at 16384 planes of 55 x 55: 160 -> 136 us; smaller
+                            // sizes got slower)
+                            const floatx4_nt t = __builtin_nontemporal_load(reinterpret_cast<const floatx4_nt *>(g4 + i));
+                            q[u] = make_float4(t.x, t.y, t.z, t.w);
+                        } else {
+                            q[u] = g4[i];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int i = i0 + NT * u;
+                    if (i < n4) {
+                        const float v[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+                        int r_ = row, x_ = x;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            smem[r_ * LDR + padL + x_] = v[c];
+                            if (++x_ == w) { x_ = 0; ++r_; }
+                        }
+                    }
+                    row += drow;
+                    x += dx;
+                    if (x >= w) { x -= w; ++row; }
+                }
+            }
+        } else {
+            for (int i = tid; i < n4; i += NT) {
+                float v[4];
+                int r_ = row, x_ = x;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    v[c] = smem[r_ * LDR + padL + x_];
+                    if (++x_ == w) { x_ = 0; ++r_; }
+                }
+                store_nt(g4 + i, make_float4(v[0], v[1], v[2], v[3]));
+                row += drow;
+                x += dx;
+                if (x >= w) { x -= w; ++row; }
+            }
+        }
+        done = n4 << 2;
+    }
+    {
+        const int first = done + tid;
+        int row = first / w, x = first - row * w;
+        const int drow = NT / w, dx = NT - drow * w;
+        for (int i = first; i < total; i += NT) {
+            float *sp = smem + row * LDR + padL + x;
+            if (TO_LDS) *sp = g[i]; else g[i] = *sp;
+            row += drow;
+            x += dx;
+            if (x >= w) { x -= w; ++row; }
+        }
+    }
+}
+
+// Spectrum stores.  Runs of whole 128-byte lines (N <= 32) are streamed past the cache (measured: 8.3 ->
+// 6.9 us for the 16384-plane N = 16 transform); the half-line runs of N >= 64 rely on the L2 to join the
+// two workgroups that share a line and stay ordinary stores.
+template <bool WHOLE_LINES>
+__device__ __forceinline__ void store_freq_run(float2 *p, const float2 &v)
+{
+    if constexpr (WHOLE_LINES) store_nt(p, v);
+    else *p = v;
+}
+
+// Raw staging for the forward transform: the chunk of nfloats contiguous floats at g goes to LDS as it
+// lies, by LDS-direct loads (global_load_lds): no staging registers, no LDS store instructions and no
+// index arithmetic; the row pass then reads its rows at their (unaligned) places and masks the padding.
+// 16-byte pieces where the chunk allows (aligned16), 4-byte pieces for the rest.  The destination of a
+// wave instruction is wave-uniform; lane l lands at + l * size.  AUX: cache policy bits (2 = non-temporal).
+template <int AUX, int NT = 256>
+__device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloats, bool aligned16, int tid)
+{
+    const int wave = tid >> 6, lane = tid & 63;
+    int done = 0;
+    if (aligned16) {
+        const int n16 = nfloats >> 2;
+        for (int p0 = wave * 64; p0 < n16; p0 += NT) {
+            if (p0 + lane < n16)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1))) *)(g + 4 * (p0 + lane)),
+                    (void __attribute__((address_space(3))) *)(raw + 4 * p0), 16, 0, AUX);
+        }
+        done = n16 << 2;
+    }
+    for (int e0 = done + wave * 64; e0 < nfloats; e0 += NT) {
+        if (e0 + lane < nfloats)
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(g + e0 + lane),
+                                             (void __attribute__((address_space(3))) *)(raw + e0), 4, 0, AUX);
+    }
+}
+
+// Zeroes the margins of nrows canvas rows and the all-zero row kept at index zrow.
+template <int N, int NT = 256>
+__device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int w, int padL, int zrow,
+                                                    int tid)
+{
+    constexpr int LDR = Canvas<N>::LDR;
+    for (int row = tid; row < nrows; row += NT) {
+        float *sp = smem + row * LDR;
+        for (int c = 0; c < padL; ++c) sp[c] = 0.0f;
+        for (int c = padL + w; c < N; ++c) sp[c] = 0.0f;
+    }
+    if (tid < N) smem[zrow * LDR + tid] = 0.0f;
+}
+
+// One launch can transform two tensors of the same FFT size (the two forward FFTs of a pass):
+// workgroups [0, blocks0) work on job 0, the rest on job 1.
+struct FwdJob {
+    const float *in;
+    float2 *out;
+    long planes;
+    int h, w, padU, padL, vec4;
+    int tbl_off;  // windowed operand: float offset of the window table in LDS
+    int herm;     // leave out the entries (ky > N/2, kx in {0, N/2}): conjugates of (N - ky, kx)
+    Window win;
+};
+
+}  // namespace fbfc

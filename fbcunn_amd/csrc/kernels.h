@@ -64,6 +64,11 @@ long fft_max_planes(int N);
 // After it no launch makes an attribute call (launches may be captured whatever shape comes first).
 hipError_t fft_prepare_device();
 
+// fft_large.hip: the transforms of size 64 and 128 (plain operands; no windows)
+hipError_t launch_rfft2d_large(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s);
+hipError_t launch_irfft2d_large(int N, const InvArgs &a, hipStream_t s);
+hipError_t fft_large_prepare_device();
+
 // fft_small.hip ------------------------------------------------------------------
 // 1-D batched transforms, N in {2,4,...,128}: rows of n reals at pad_l of the N-point canvas
 // <-> (rows, N/2+1) complex, row-major; the inverse is unnormalised.
