@@ -10,8 +10,19 @@ resident in HBM before the timed region starts.  `value` is the effective
 convolution rate: direct-convolution FLOPs (2*B*F*P*oH*oW*kH*kW per pass, three
 passes per step) divided by wall time.  The line also carries ms per pass, the
 roofline position of every stage (HIP events recorded by the library on the
-stream its kernels run on), the dominant kernel's roofline object and the CPU
-oracle timed on this box's host cores.
+stream its kernels run on), the dominant kernel's roofline object, the CPU
+oracle timed on this box's host cores and, under "configs", the same per-pass and
+per-stage records for the other stated configurations (the 8192-plane FFT round
+trip, the batch-128 updateOutput layer and the large-kernel layer).
+
+Every stage is timed twice: `ms` is the mean of STAGE_REPS back-to-back launches
+between two events (inputs warm in the caches, no event overhead), `ms_single`
+the median of single launches inside an ordinary pass, one event pair around each
+(about 2 us of event overhead included).  Roofline fractions use `ms`.  For the
+contraction, `algorithmic_frac` counts 8 flops per complex multiply-add and
+`mfma_issued_frac` the 6 the kernels issue (three real products per complex one):
+the second is the utilisation of the fp32 matrix pipe.  Kernel names and grids come
+from the library (fbfc_plan_stage_kernel), as a profiler trace shows them.
 """
 import argparse
 import json
@@ -62,44 +73,35 @@ def stage_model(cfg, pass_, n, q):
             "ifft": ("hbm", fft(F * P, k) + 8 * B * F)}
 
 
-# HBM bytes per launch at the main workload, from the committed rocprofv3 --pmc runs
-# (profiles/hbm_traffic_all_configs.txt): FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, the
-# factors a 256 MiB device copy gives for the same counters (--calibrate-copy).
-MEASURED_TRAFFIC_MAIN = {
-    "cgemm_hybrid_kernel<0>": (17091 * 2.0 + 16642) * 1024,
-    "cgemm_hybrid_kernel<1>": (17096 * 2.0 + 16642) * 1024,
-    "cgemm_hybrid_kernel<2>": (17096 * 2.0 + 16641) * 1024,
-}
-
-KERNEL_OF_STAGE = {"fft": "rfft2d_kernel", "mm": "cgemm_freq_kernel", "ifft": "irfft2d_kernel"}
+TRAFFIC_PROFILE = os.path.join("profiles", "hbm_traffic_all_configs.txt")
 
 
-def mm_kernel_name(pass_, q, m, n, k):
-    """Which contraction kernel the library picks (the rule of launch_mode in
-    fbcunn_amd/csrc/cgemm_kernels.hip), so that the stage table names the kernel
-    a rocprofv3 trace of the same run shows."""
-    mode = {"fprop": 0, "bprop": 1, "accgrad": 2}[pass_]
-    tiles64 = q * ((m + 63) // 64) * ((n + 63) // 64)
-    direct_ok = m % 64 == 0 and n % 64 == 0 and k % 16 == 0
-    if direct_ok and k % 64 == 0 and 256 <= tiles64 < 8 * 256 and tiles64 % 256 <= 128:
-        t64 = (m // 64) * (n // 64)
-        q_direct = (tiles64 // 256) * 256 // t64
-        if 0 < q_direct < q:
-            return "cgemm_hybrid_kernel<%d>" % mode
-    if mode != 1 and m % 64 == 0 and n % 96 == 0 and n % 64 != 0 and k % 16 == 0 and q * (m // 64) * (n // 96) >= 4 * 256:
-        return "cgemm_ldsdirect_kernel<%d, 3>" % mode
-    if direct_ok and tiles64 >= 4 * 256:
-        return "cgemm_ldsdirect_kernel<%d, 2>" % mode
-    if m % 32 == 0 and n % 32 == 0 and k % 16 == 0:
-        tot32 = q * (m // 32) * (n // 32)
-        if tot32 < 4096 and k % 64 == 0:
-            return "cgemm_splitk_kernel<%d, 4>" % mode
-        if tot32 < 8192 and k % 32 == 0:
-            return "cgemm_splitk_kernel<%d, 2>" % mode
-        return "cgemm_splitk_kernel<%d, 1>" % mode
-    if direct_ok:
-        return "cgemm_ldsdirect_kernel<%d, 2>" % mode
-    return "cgemm_freq_kernel<%d>" % mode
+def profiled_traffic():
+    """HBM bytes per launch, per (kernel, grid), from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, the factors a 256 MiB device copy gives for the
+    same counters).  Empty if the file is missing."""
+    import re
+    out = {}
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+    except OSError:
+        return out
+    pat = re.compile(r"^(?:fbfc::)?(\S.*?)\s+grid=(\d+)\s+FETCH_SIZE=(\d+) KiB \(x([0-9.]+).*?WRITE_SIZE=(\d+) KiB \(x([0-9.]+)", re.M)
+    for m in pat.finditer(text):
+        name, grid = m.group(1).strip(), int(m.group(2))
+        out[(name, grid)] = (int(m.group(3)) * float(m.group(4)) + int(m.group(5)) * float(m.group(6))) * 1024
+    return out
+
+
+def split_launch(desc):
+    """'<kernel> grid=<n>; ...' -> [(kernel, grid), ...]"""
+    out = []
+    for part in desc.split(";"):
+        part = part.strip()
+        if part:
+            name, _, grid = part.rpartition(" grid=")
+            out.append((name, int(grid)))
+    return out
 
 
 def make_layer(nn, torch, synth, cfg):
@@ -148,6 +150,29 @@ def time_each(torch, fn, steps, warmup):
     return {"median": ms[len(ms) // 2], "min": ms[0]}
 
 
+def stage_times(net, x, g, p, reps, runs):
+    """Per-stage ms of pass p with `reps` back-to-back launches per stage, and what each stage
+    launched.  Mean over `runs` passes for reps > 1, median for reps == 1."""
+    net.timed = reps
+    acc, kernels = {}, {}
+    run_pass(net, x, g, p)
+    for _ in range(runs):
+        run_pass(net, x, g, p)
+        one = {}
+        for s, v in net.stageTimes(x).items():
+            s = "fft" if s in ("fft_a", "fft_b") else s   # the forward transforms of the pass
+            one[s] = one.get(s, 0.0) + v
+        for s, v in one.items():
+            acc.setdefault(s, []).append(v)
+    for s, v in net.stageKernels(x).items():
+        s = "fft" if s in ("fft_a", "fft_b") else s
+        kernels[s] = (kernels[s] + "; " + v) if s in kernels else v
+    net.timed = False
+    if reps > 1:
+        return {s: sum(v) / len(v) for s, v in acc.items()}, kernels
+    return {s: sorted(v)[len(v) // 2] for s, v in acc.items()}, kernels
+
+
 def measure_config(nn, torch, synth, name, steps, warmup):
     cfg = CONFIGS[name]
     B, P, F, H, k, pad, passes = cfg[:7]
@@ -168,51 +193,47 @@ def measure_config(nn, torch, synth, name, steps, warmup):
         entry = {"ms": ms, "effective_tflops": flop_pass / (ms * 1e-3) / 1e12,
                  "ms_single_call": time_each(torch, lambda: run_pass(net, x, g, p), max(10, steps), warmup),
                  "stages": {}}
-        # per-stage HIP-event timing: the library launches each stage STAGE_REPS times back to back
-        # between two events on the pass's stream, so the event overhead (about 2 us) does not
-        # inflate kernels that only run for 5-10 us
-        net.timed = STAGE_REPS
-        acc = {}
-        reps = 3
-        run_pass(net, x, g, p)
-        for _ in range(reps):
-            run_pass(net, x, g, p)
-            for s, v in net.stageTimes(x).items():
-                s = "fft" if s in ("fft_a", "fft_b") else s   # one launch for both operands
-                acc[s] = acc.get(s, 0.0) + v
-        net.timed = False
+        warm, kernels = stage_times(net, x, g, p, STAGE_REPS, 3)
+        single, _ = stage_times(net, x, g, p, 1, 7)
         model = stage_model(cfg, p, n, q)
         for s, spec in model.items():
-            ms_s = acc.get(s, 0.0) / reps
+            ms_s = warm.get(s, 0.0)
             if ms_s <= 0:
                 continue
+            st = {"kernel": kernels.get(s, ""), "ms": ms_s, "ms_single": single.get(s), "bound": spec[0]}
             if spec[0] == "hbm":
                 ach = spec[1] / (ms_s * 1e-3) / 1e9
-                entry["stages"][s] = {"kernel": KERNEL_OF_STAGE[s], "ms": ms_s, "bound": "hbm",
-                                      "bytes": spec[1], "achieved": ach, "unit": "GB/s",
-                                      "peak": HBM_PEAK_GBS, "frac": ach / HBM_PEAK_GBS}
+                st.update({"bytes": spec[1], "achieved": ach, "unit": "GB/s", "peak": HBM_PEAK_GBS,
+                           "frac": ach / HBM_PEAK_GBS})
             else:
                 ach = spec[1] / (ms_s * 1e-3) / 1e12
-                mnk = {"fprop": (B, F, P), "bprop": (B, P, F), "accgrad": (F, P, B)}[p]
-                kname = mm_kernel_name(p, q - (n - 2), *mnk)
                 # the kernels form a complex product from three real ones: they issue 6 of the
                 # 8 algorithmic flops per complex multiply-add
                 issued = spec[1] * 0.75
-                entry["stages"][s] = {"kernel": kname, "ms": ms_s, "bound": "mfma",
-                                      "flops": spec[1], "bytes": spec[2], "achieved": ach,
-                                      "unit": "TFLOP/s", "peak": MFMA_FP32_PEAK_TF,
-                                      "frac": ach / MFMA_FP32_PEAK_TF,
-                                      "flops_issued": issued,
-                                      "issued_frac": issued / (ms_s * 1e-3) / 1e12 / MFMA_FP32_PEAK_TF,
-                                      "hbm_gbs": spec[2] / (ms_s * 1e-3) / 1e9}
+                st.update({"flops": spec[1], "bytes": spec[2], "achieved": ach, "unit": "TFLOP/s",
+                           "peak": MFMA_FP32_PEAK_TF, "frac": ach / MFMA_FP32_PEAK_TF,
+                           "algorithmic_frac": ach / MFMA_FP32_PEAK_TF, "flops_issued": issued,
+                           "mfma_issued_frac": issued / (ms_s * 1e-3) / 1e12 / MFMA_FP32_PEAK_TF,
+                           "hbm_gbs": spec[2] / (ms_s * 1e-3) / 1e9})
+            entry["stages"][s] = st
         res["passes"][p] = entry
     res["fft_size"] = n
     net.cleanupBuffers()
     return res
 
 
+def compact(res):
+    """The per-pass / per-stage record of a configuration without the byte and flop counts."""
+    keep = ("kernel", "ms", "ms_single", "bound", "frac", "algorithmic_frac", "mfma_issued_frac")
+    return {"ms_per_step": res["ms_per_step"], "effective_tflops": res["effective_tflops"], "fft_size": res["fft_size"],
+            "passes": {p: {"ms": e["ms"], "effective_tflops": e["effective_tflops"],
+                           "stages": {s: {k: st[k] for k in keep if k in st} for s, st in e["stages"].items()}}
+                       for p, e in res["passes"].items()}}
+
+
 def measure_fft_round_trip(nn, torch, synth, steps, warmup):
-    """8192 planes of 32x32: forward then inverse, each timed on its own."""
+    """8192 planes of 32x32: forward then inverse, each timed on its own (`ms`: back-to-back
+    launches between two events; `ms_single`: median of single launches, an event pair around each)."""
     n, planes = 32, 8192
     x = torch.from_numpy(synth.uniform(1002, (planes, n, n))).cuda()
     freq = torch.empty((n, n // 2 + 1, planes, 2), device="cuda")
@@ -231,7 +252,8 @@ def measure_fft_round_trip(nn, torch, synth, steps, warmup):
         ms = ev0.elapsed_time(ev1) / steps
         nbytes = 4 * planes * n * n + 8 * planes * n * (n // 2 + 1)
         ach = nbytes / (ms * 1e-3) / 1e9
-        out[name] = {"ms": ms, "bytes": nbytes, "achieved": ach, "unit": "GB/s", "peak": HBM_PEAK_GBS,
+        out[name] = {"kernel": w.lastKernel(), "ms": ms, "ms_single": time_each(torch, fn, 15, 2)["median"],
+                     "bound": "hbm", "bytes": nbytes, "achieved": ach, "unit": "GB/s", "peak": HBM_PEAK_GBS,
                      "frac": ach / HBM_PEAK_GBS}
     return out
 
@@ -387,7 +409,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--all-configs", action="store_true", help="also measure configs 2, 3 and 5")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also measure the tiled VGG-like layer and the reference's benchmark layers")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run a plain 256 MiB device copy 3 times (a kernel of known traffic "
@@ -419,12 +442,22 @@ def main():
             if st["ms"] > worst_ms:
                 worst, worst_ms = (p, s, st), st["ms"]
     p, s, st = worst
+    traffic = None
+    launches = split_launch(st["kernel"])
+    table = profiled_traffic()
+    if len(launches) == 1 and launches[0] in table:
+        traffic = table[launches[0]]
     roofline = {"bound": st["bound"], "achieved": st["achieved"], "peak": st["peak"], "unit": st["unit"],
-                "frac": st["frac"], "traffic": MEASURED_TRAFFIC_MAIN.get(st["kernel"]), "kernel": st["kernel"], "pass": p, "stage": s,
-                "avg_launch_ms": st["ms"]}
-    if "issued_frac" in st:
-        # achieved counts the algorithmic 8 flops per complex multiply-add; the kernel issues 6 of them
-        roofline["issued_frac"] = st["issued_frac"]
+                "frac": st["frac"], "traffic": traffic,
+                "traffic_source": (TRAFFIC_PROFILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel and grid; "
+                                   "not measured in this run)") if traffic is not None else None,
+                "kernel": st["kernel"], "pass": p, "stage": s, "avg_launch_ms": st["ms"],
+                "single_launch_ms": st["ms_single"]}
+    if "mfma_issued_frac" in st:
+        # achieved / frac count the algorithmic 8 flops per complex multiply-add; the kernel issues 6 of
+        # them: mfma_issued_frac is the utilisation of the fp32 matrix pipe
+        roofline["algorithmic_frac"] = st["algorithmic_frac"]
+        roofline["mfma_issued_frac"] = st["mfma_issued_frac"]
 
     line = {
         "metric": "effective conv TFLOP/s (direct-convolution FLOPs / time), full training step at batch 128",
@@ -443,15 +476,17 @@ def main():
     line["reuse_all_step"] = measure_reuse_step(nn, torch, synth, args.steps, args.warmup)
     line["fprop_plus_backward_step"] = measure_backward_step(nn, torch, synth, args.steps, args.warmup)
     line["copy_256MiB"] = measure_copy_bandwidth(torch)
+    # the other stated configurations, compact
+    configs = {}
+    for name in CONFIGS:
+        if name != MAIN:
+            configs[name] = compact(measure_config(nn, torch, synth, name, max(5, args.steps // 5), 2))
+    configs["config2_fft_round_trip_8192x32x32"] = measure_fft_round_trip(nn, torch, synth, args.steps, args.warmup)
+    line["configs"] = configs
     if args.all_configs:
-        others = {}
-        for name in CONFIGS:
-            if name != MAIN:
-                others[name] = measure_config(nn, torch, synth, name, max(5, args.steps // 5), 2)
-        others["config2_fft_round_trip_8192x32x32"] = measure_fft_round_trip(nn, torch, synth, args.steps, args.warmup)
-        others["tiled_convolution"] = measure_tiled(nn, torch, synth, args.steps, args.warmup)
-        others["reference_benchmark_layers"] = measure_reference_list(nn, torch, synth, args.steps)
-        line["other_configs"] = others
+        line["other_workloads"] = {
+            "tiled_convolution": measure_tiled(nn, torch, synth, args.steps, args.warmup),
+            "reference_benchmark_layers": measure_reference_list(nn, torch, synth, args.steps)}
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)
     print(json.dumps(line))
 

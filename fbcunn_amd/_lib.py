@@ -45,6 +45,7 @@ _vp, _i, _f, _l = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
 SIGNATURES = {
     "fbfc_version": (ctypes.c_char_p, []),
     "fbfc_last_error": (ctypes.c_char_p, []),
+    "fbfc_last_launch": (ctypes.c_char_p, []),
     "fbfc_plan_query": (_i, [ctypes.POINTER(ConvDesc), ctypes.POINTER(PlanInfo)]),
     "fbfc_plan_create": (_i, [ctypes.POINTER(ConvDesc), ctypes.POINTER(_vp)]),
     "fbfc_plan_query_tiled": (_i, [ctypes.POINTER(ConvDesc), _i, _i, ctypes.POINTER(PlanInfo)]),
@@ -58,7 +59,7 @@ SIGNATURES = {
     "fbfc_plan_set_reuse": (_i, [_vp, ctypes.c_uint]),
     "fbfc_plan_set_timed": (_i, [_vp, _i]),
     "fbfc_plan_stage_ms": (_i, [_vp, ctypes.POINTER(_f), _i]),
-    "fbfc_plan_contraction_kernel": (_i, [_vp, ctypes.c_char_p, ctypes.c_size_t]),
+    "fbfc_plan_stage_kernel": (_i, [_vp, _i, ctypes.c_char_p, ctypes.c_size_t]),
     "fbfc_debug_force_contraction_kernel": (_i, [_i]),
     "fbfc_fft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp]),
     "fbfc_ifft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),

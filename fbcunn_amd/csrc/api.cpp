@@ -14,6 +14,20 @@
 #include "../../include/fbfftconv.h"
 #include "kernels.h"
 
+namespace fbfc {
+
+static thread_local std::string g_kernel_log;
+void kernel_log_clear() { g_kernel_log.clear(); }
+void kernel_log_add(const char *name, long grid_items)
+{
+    char buf[128];
+    std::snprintf(buf, sizeof buf, "%s%s grid=%ld", g_kernel_log.empty() ? "" : "; ", name, grid_items);
+    g_kernel_log += buf;
+}
+const char *kernel_log_get() { return g_kernel_log.c_str(); }
+
+}  // namespace fbfc
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -191,7 +205,7 @@ struct fbfc_plan {
     hipEvent_t ev[FBFC_NUM_STAGES + 1];
     bool ev_made;
     float stage_ms[FBFC_NUM_STAGES];
-    char mm_kernel[48];  // the contraction kernel the last pass launched
+    char stage_kernel[FBFC_NUM_STAGES][160];  // what each stage of the last pass launched
 };
 
 namespace {
@@ -204,6 +218,8 @@ struct StageTimer {
     int slot[FBFC_NUM_STAGES];
     StageTimer(fbfc_plan *plan, hipStream_t stream) : p(plan), s(stream), n(0)
     {
+        for (auto &name : p->stage_kernel) name[0] = 0;
+        fbfc::kernel_log_clear();
         if (p->timed) {
             for (float &m : p->stage_ms) m = 0.0f;
             (void)hipEventRecord(p->ev[0], s);
@@ -211,8 +227,16 @@ struct StageTimer {
     }
     // number of back-to-back launches of each stage (1 unless the plan is timed)
     int reps() const { return p->timed > 0 ? p->timed : 1; }
+    // after the first of several repetitions: what it logged is the stage's launch list
+    std::string first_log;
+    void keep_log() { first_log = fbfc::kernel_log_get(); }
     void done(int stage)
     {
+        // what the stage launched (once, whatever the number of timed repetitions: the first entries)
+        std::snprintf(p->stage_kernel[stage], sizeof p->stage_kernel[stage], "%s",
+                      first_log.empty() ? fbfc::kernel_log_get() : first_log.c_str());
+        first_log.clear();
+        fbfc::kernel_log_clear();
         if (!p->timed) return;
         slot[n] = stage;
         ++n;
@@ -244,6 +268,7 @@ struct StageTimer {
 #define FBFC_STAGE(tm, expr, what)                             \
     do {                                                       \
         for (int r_ = 0; r_ < (tm).reps(); ++r_) {             \
+            if (r_ == 1) (tm).keep_log();                      \
             hipError_t e_ = (expr);                            \
             if (e_ != hipSuccess) return fail_hip(e_, what);   \
         }                                                      \
@@ -317,6 +342,8 @@ extern "C" {
 const char *fbfc_version(void) { return "fbfftconv 0.1 (gfx950)"; }
 
 const char *fbfc_last_error(void) { return g_last_error.c_str(); }
+
+const char *fbfc_last_launch(void) { return fbfc::kernel_log_get(); }
 
 int fbfc_plan_query(const fbfc_conv_desc *desc, fbfc_plan_info *info)
 {
@@ -424,10 +451,11 @@ int fbfc_plan_set_timed(fbfc_plan *p, int on)
     return FBFC_OK;
 }
 
-int fbfc_plan_contraction_kernel(const fbfc_plan *p, char *name, size_t n)
+int fbfc_plan_stage_kernel(const fbfc_plan *p, int stage, char *name, size_t n)
 {
     if (p == nullptr || name == nullptr || n == 0) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
-    std::snprintf(name, n, "%s", p->mm_kernel);
+    if (stage < 0 || stage >= FBFC_NUM_STAGES) return fail(FBFC_ERR_INVALID_ARGUMENT, "no such stage");
+    std::snprintf(name, n, "%s", p->stage_kernel[stage]);
     return FBFC_OK;
 }
 
@@ -482,7 +510,6 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     // O[b][f] = 1/N^2 sum_p I[b][p] conj(W[f][p])   (SpatialConvolutionFBFFT.lua:157-164)
     FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(0, p->in_freq, p->w_freq, res, QH, fm, g.vbatch, d.out_planes,
                                      d.in_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(fprop)");
-    std::snprintf(p->mm_kernel, sizeof p->mm_kernel, "%s", fbfc::cgemm_last_kernel());
     tm.done(FBFC_STAGE_MM);
     const fbfc::InvArgs inv = {res, output, (long)g.vbatch * d.out_planes, g.r_h, g.r_w, g.r_pad_u, g.r_pad_l,
                                bias, d.out_planes, g.r_win, nullptr, nullptr, 0.0f, 0, 0};
@@ -523,7 +550,6 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     // GI[b][p] = 1/N^2 sum_f GO[b][f] W[f][p]   (SpatialConvolutionFBFFT.lua:244-251)
     FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(1, p->out_freq, p->w_freq, res, QH, fm, g.vbatch, d.in_planes,
                                      d.out_planes, 1.0f / ((float)N * (float)N), 0, s), "cgemm(bprop)");
-    std::snprintf(p->mm_kernel, sizeof p->mm_kernel, "%s", fbfc::cgemm_last_kernel());
     tm.done(FBFC_STAGE_MM);
     const fbfc::InvArgs inv = {res, grad_input, (long)g.vbatch * d.in_planes, g.r_h, g.r_w, g.r_pad_u,
                                g.r_pad_l, nullptr, 1, g.r_win, nullptr, nullptr, 0.0f, 0, 0};
@@ -570,7 +596,6 @@ static int acc_grad_parameters(fbfc_plan *p, const float *input, const float *gr
     // GW[f][p] = scale/N^2 sum_b conj(GO[b][f]) I[b][p]   (SpatialConvolutionFBFFT.lua:337-344)
     FBFC_STAGE(tm, fbfc::launch_cgemm_freq_map(2, p->out_freq, p->in_freq, res, QH, fm, d.out_planes, d.in_planes,
                                      g.vbatch, scale / ((float)N * (float)N), 0, s), "cgemm(accGrad)");
-    std::snprintf(p->mm_kernel, sizeof p->mm_kernel, "%s", fbfc::cgemm_last_kernel());
     tm.done(FBFC_STAGE_MM);
     fbfc::InvArgs inv = {res, grad_weight, (long)d.out_planes * d.in_planes, g.r_h, g.r_w, 0, 0, nullptr, 1, {},
                          nullptr, nullptr, 0.0f, 0, 0};
@@ -610,6 +635,7 @@ int fbfc_backward(fbfc_plan *p, const float *input, const float *grad_output, co
 int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
                float *freq, void *stream)
 {
+    fbfc::kernel_log_clear();
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
         return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
@@ -630,6 +656,7 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
 int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
                 float *real, const float *bias, int bias_period, void *stream)
 {
+    fbfc::kernel_log_clear();
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
         return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
@@ -652,6 +679,7 @@ static bool fft1d_size_ok(int n) { return n >= 2 && n <= 128 && (n & (n - 1)) ==
 
 int fbfc_fft1d(const float *real, long rows, int n, int pad_l, int fft_size, float *freq, void *stream)
 {
+    fbfc::kernel_log_clear();
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (!fft1d_size_ok(fft_size)) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
     if (rows < 1 || n < 1 || pad_l < 0 || n + pad_l > fft_size)
@@ -663,6 +691,7 @@ int fbfc_fft1d(const float *real, long rows, int n, int pad_l, int fft_size, flo
 
 int fbfc_ifft1d(const float *freq, long rows, int n, int pad_l, int fft_size, float *real, void *stream)
 {
+    fbfc::kernel_log_clear();
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (!fft1d_size_ok(fft_size)) return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
     if (rows < 1 || n < 1 || pad_l < 0 || n + pad_l > fft_size)
@@ -675,6 +704,7 @@ int fbfc_ifft1d(const float *freq, long rows, int n, int pad_l, int fft_size, fl
 int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq, int m, int n, int k,
                       float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate, void *stream)
 {
+    fbfc::kernel_log_clear();
     if (A == nullptr || B == nullptr || C == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (n_freq < 1 || m < 1 || n < 1 || k < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
     if (conj_trans_a && conj_trans_b)

@@ -622,6 +622,14 @@ __global__ __launch_bounds__(256) void cgemm_hybrid_kernel(const float2 *__restr
     }
 }
 
+static void note_kernel(const char *base, int mode, int variant, long grid_items)
+{
+    char name[64];
+    if (variant >= 0) snprintf(name, sizeof name, "%s<%d, %d>", base, mode, variant);
+    else snprintf(name, sizeof name, "%s<%d>", base, mode);
+    kernel_log_add(name, grid_items);
+}
+
 template <int MODE, int SK>
 static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_freq, int m, int n,
                                 int k, float alpha, int accumulate, FreqMap fm, hipStream_t s)
@@ -630,6 +638,7 @@ static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_
     const long tot32 = (long)n_freq * tm * tn;
     const long wgs = (tot32 * SK + 3) / 4;
     const int chunk = (int)((wgs + 7) / 8);
+    note_kernel("cgemm_splitk_kernel", MODE, SK, (long)chunk * 8 * 256);
     hipLaunchKernelGGL((cgemm_splitk_kernel<MODE, SK>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                        reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tm, tn, (int)tot32,
@@ -644,14 +653,6 @@ static std::atomic<int> g_force_variant{-1};
 void cgemm_force_variant(int v) { g_force_variant.store(v); }
 static int splitk_override() { return g_force_variant.load(std::memory_order_relaxed); }
 
-// name of the kernel the last contraction launched from this thread chose
-static thread_local char g_last_kernel[48] = "";
-const char *cgemm_last_kernel() { return g_last_kernel; }
-static void note_kernel(const char *base, int mode, int variant)
-{
-    if (variant >= 0) snprintf(g_last_kernel, sizeof g_last_kernel, "%s<%d, %d>", base, mode, variant);
-    else snprintf(g_last_kernel, sizeof g_last_kernel, "%s<%d>", base, mode);
-}
 
 template <int MODE>
 static hipError_t launch_mode(const float *A, const float *B, float *C, int n_freq, int m, int n,
@@ -681,7 +682,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
             const int direct_wgs = q_direct * t64;
             const int split_tiles = q_split * (m / 32) * (n / 32);  // one workgroup per 32x32 block
             const int chunk_direct = (direct_wgs + 7) / 8, chunk_split = (split_tiles + 7) / 8;
-            note_kernel("cgemm_hybrid_kernel", MODE, -1);
+            note_kernel("cgemm_hybrid_kernel", MODE, -1, (long)(chunk_direct + chunk_split) * 8 * 256);
             hipLaunchKernelGGL(cgemm_hybrid_kernel<MODE>, dim3((unsigned)((chunk_direct + chunk_split) * 8)),
                                dim3(256), 0, s, reinterpret_cast<const float2 *>(A),
                                reinterpret_cast<const float2 *>(B), reinterpret_cast<float2 *>(C), m, n, k,
@@ -698,7 +699,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
         const int t96 = n / 96;
         const long tot = (long)n_freq * tilesM * t96;
         const int ch = (int)((tot + 7) / 8);
-        note_kernel("cgemm_ldsdirect_kernel", MODE, 3);
+        note_kernel("cgemm_ldsdirect_kernel", MODE, 3, (long)ch * 8 * 384);
         hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 3>), dim3((unsigned)(ch * 8)), dim3(384), 0, s,
                            reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                            reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, t96, (int)tot, ch,
@@ -713,21 +714,20 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
         else if (tot32 < 4 * 1024 && (k % 64) == 0) sk = 4;
         else if (tot32 < 8 * 1024 && (k % 32) == 0) sk = 2;
         else sk = 1;
-        if ((sk == 4 && (k % 64) == 0) || (sk == 2 && (k % 32) == 0) || sk == 1) note_kernel("cgemm_splitk_kernel", MODE, sk);
-        if (sk == 4 && (k % 64) == 0) return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+                if (sk == 4 && (k % 64) == 0) return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
         if (sk == 2 && (k % 32) == 0) return launch_splitk<MODE, 2>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
         if (sk == 1) return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
     }
     const int chunk = (int)((total + 7) / 8);
     if (direct_ok && force != 0) {
-        note_kernel("cgemm_ldsdirect_kernel", MODE, 2);
+        note_kernel("cgemm_ldsdirect_kernel", MODE, 2, (long)chunk * 8 * 256);
         hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 2>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                            reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                            reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
                            (int)total, chunk, fm);
         return hipGetLastError();
     }
-    note_kernel("cgemm_freq_kernel", MODE, -1);
+    note_kernel("cgemm_freq_kernel", MODE, -1, (long)chunk * 8 * 256);
     hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                        reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,

@@ -22,6 +22,7 @@
 // The inverse kernel is the mirror image and adds the bias while cropping.
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
 #include <mutex>
 
 #include "bias_dc.h"
@@ -636,6 +637,11 @@ static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipSt
         lds += FftShape<N>::T * sizeof(int4);
     }
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    {
+        char name[64];
+        snprintf(name, sizeof name, "rfft2d_kernel<%d, %s, %d, %s>", N, WIN ? "true" : "false", NZ, RAW ? "true" : "false");
+        kernel_log_add(name, blocks * FftShape<N, false, (NZ < N)>::THREADS);
+    }
     hipLaunchKernelGGL((rfft2d_kernel<N, WIN, NZ, RAW>), dim3((unsigned)blocks), dim3(FftShape<N, false, (NZ < N)>::THREADS), lds, s, j0, j1,
                        (unsigned)blocks0);
     return hipGetLastError();
@@ -667,6 +673,11 @@ static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s)
                                a.out_planes};
     const unsigned bblocks = (bgrad.dc != nullptr) ? bias_grad_dc_blocks(bgrad.planes) : 0u;
     if (blocks + bblocks > 0x7fffffffL) return hipErrorInvalidValue;
+    {
+        char name[64];
+        snprintf(name, sizeof name, "irfft2d_kernel<%d, %s, %d>", N, WIN ? "true" : "false", PHASES);
+        kernel_log_add(name, (blocks + bblocks) * S::THREADS);
+    }
     hipLaunchKernelGGL((irfft2d_kernel<N, WIN, PHASES>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
                        reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL,
                        a.bias, a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks, win, tbl_off);

@@ -21,6 +21,8 @@
 // 256 registers; 512 at N = 128 with T = 4, where a lane held 256 values and spilled.
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
+
 #include "bias_dc.h"
 #include "fft_regs.h"
 #include "fft_stage.h"
@@ -511,6 +513,11 @@ static hipError_t launch_fwd_rows(const FwdArgs &a, const FwdArgs *second, hipSt
         j1 = make_rows_job<N, T, SMALL>(*second);
     }
     if (blocks > 0x7fffffffL || lds > 160 * 1024) return hipErrorInvalidValue;
+    {
+        char name[64];
+        snprintf(name, sizeof name, "rfft2d_rows_kernel<%d, %d, %d, %s>", N, T, NZ, RAW ? "true" : "false");
+        kernel_log_add(name, blocks * S::THREADS);
+    }
     hipLaunchKernelGGL((rfft2d_rows_kernel<N, T, NZ, RAW>), dim3((unsigned)blocks), dim3(S::THREADS), lds, s, j0, j1,
                        (unsigned)blocks0);
     return hipGetLastError();
@@ -528,6 +535,11 @@ static hipError_t launch_inv_rows(const InvArgs &a, hipStream_t s)
                                a.out_planes};
     const unsigned bblocks = (bgrad.dc != nullptr) ? bias_grad_dc_blocks(bgrad.planes) : 0u;
     if (blocks + bblocks > 0x7fffffffL || lds > 160 * 1024) return hipErrorInvalidValue;
+    {
+        char name[64];
+        snprintf(name, sizeof name, "irfft2d_rows_kernel<%d, %d>", N, T);
+        kernel_log_add(name, (blocks + bblocks) * S::THREADS);
+    }
     hipLaunchKernelGGL((irfft2d_rows_kernel<N, T>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
                        reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL, a.bias,
                        a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks);

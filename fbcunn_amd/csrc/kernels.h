@@ -102,8 +102,11 @@ inline int hermitian_count(int N) { return (N / 2 + 1) * (N / 2 + 1) + (N / 2 - 
 hipError_t launch_cgemm_freq_map(int mode, const float *A, const float *B, float *C, int n_freq, FreqMap fm,
                                  int m, int n, int k, float alpha, int accumulate, hipStream_t s);
 
-// Name of the kernel the last contraction launched from the calling thread chose ("" before the first).
-const char *cgemm_last_kernel();
+// Launch log of the calling thread: every kernel launcher appends "<kernel name> grid=<work-items>";
+// the pass entry points clear it before a stage and keep what the stage logged.
+void kernel_log_clear();
+void kernel_log_add(const char *name, long grid_items);
+const char *kernel_log_get();
 // Measurement knob: -1 = choose by shape; 0 = register-staged LDS tiles, 8 = LDS-direct tiles,
 // 9 = hybrid of LDS-direct tiles and split blocks, 1 / 2 / 4 = register-fed kernel with that many
 // waves per block (falls back to the shape rule where the forced variant cannot run the shape).

@@ -151,12 +151,16 @@ class SpatialConvolutionFFT:
         if input.size(1) != self.nInputPlane:
             raise ValueError("input has %d planes, module expects %d" % (input.size(1), self.nInputPlane))
 
-    def contractionKernel(self, input):
-        """Name of the contraction kernel the last pass on this input shape launched."""
+    def stageKernels(self, input):
+        """What each stage of the last pass on this input shape launched (dict stage -> string)."""
         plan = self._plan_for(input.size(0), input.size(2), input.size(3))
-        buf = ctypes.create_string_buffer(64)
-        check(lib().fbfc_plan_contraction_kernel(plan.handle, buf, len(buf)))
-        return buf.value.decode()
+        out = {}
+        for i, name in enumerate(_lib.STAGE_NAMES):
+            buf = ctypes.create_string_buffer(200)
+            check(lib().fbfc_plan_stage_kernel(plan.handle, i, buf, len(buf)))
+            if buf.value:
+                out[name] = buf.value.decode()
+        return out
 
     def stageTimes(self, input):
         """Mean ms per launch of each stage of the last pass run with self.timed = reps > 0 (dict)."""
@@ -313,6 +317,10 @@ class FFTWrapper:
         if time.numel() != planes * h * w:
             raise ValueError("time and frequency disagree on the number of planes")
         return 2, n, planes, h, w
+
+    def lastKernel(self):
+        """What the last transform called from this thread launched ("<kernel> grid=<work-items>")."""
+        return lib().fbfc_last_launch().decode()
 
     def _run(self, call, dims, n, batches):
         if not self.timed:

@@ -69,6 +69,12 @@ const char *fbfc_version(void);
 /* Message of the last failure on this thread ("" if none). */
 const char *fbfc_last_error(void);
 
+/* What the last stand-alone transform or contraction called from this thread launched:
+ * "<kernel name> grid=<work-items>", several launches joined by "; ".  (For the passes of a plan see
+ * fbfc_plan_stage_kernel.)  Counterpart of the log line of the reference's timed wrappers
+ * (src/fft/FFTWrapperLua.cpp:137-152). */
+const char *fbfc_last_launch(void);
+
 /* Planning (host only; no GPU needed) ----------------------------------------
  * Validates the descriptor the way the module constructor and the FFT-size
  * choice do (stride 1: SpatialConvolutionFFT.lua:176, SpatialConvolutionFBFFT.lua:60-61;
@@ -157,11 +163,11 @@ enum { FBFC_STAGE_FFT_A = 0,   /* the forward-FFT launch: both operands of the p
 int fbfc_plan_set_timed(fbfc_plan *plan, int reps);
 /* Milliseconds of each stage of the last timed pass (0 for a stage not run). */
 int fbfc_plan_stage_ms(const fbfc_plan *plan, float *ms, int n);
-/* Name of the contraction kernel the plan's last pass launched (the library picks one of several
- * by shape), as a profiler trace shows it, e.g. "cgemm_hybrid_kernel<0>"; "" before the first pass.
- * The counterpart of the kernel names the reference's timed wrappers log
- * (src/CuBLASWrapperLua.cpp:39-137). */
-int fbfc_plan_contraction_kernel(const fbfc_plan *plan, char *name, size_t n);
+/* What a stage of the plan's last pass launched, as a profiler trace shows it:
+ * "<kernel name> grid=<work-items>", several launches joined by "; " ("" for a stage not run).  The
+ * library picks its kernels by shape; this is the counterpart of the names the reference's timed
+ * wrappers log (src/CuBLASWrapperLua.cpp:39-137, src/fft/FFTWrapperLua.cpp:137-152). */
+int fbfc_plan_stage_kernel(const fbfc_plan *plan, int stage, char *name, size_t n);
 /* Measurement knob (no counterpart in the reference): forces the contraction kernel variant for the
  * whole process.  -1 = choose by shape (default); 0 = register-staged LDS tiles with bounds checks,
  * 8 = LDS-direct tiles, 9 = LDS-direct tiles plus split blocks, 1 / 2 / 4 = register-fed kernel
