@@ -63,6 +63,11 @@ SIGNATURES = {
     "fbfc_debug_force_contraction_kernel": (_i, [_i]),
     "fbfc_fft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp]),
     "fbfc_ifft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
+    "fbfc_planes_layout_workspace_bytes": (ctypes.c_size_t, [_l, _i]),
+    "fbfc_fft2d_planes": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "fbfc_ifft2d_planes": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "fbfc_transpose_mm_planes_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i, _i]),
+    "fbfc_transpose_mm_planes": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _vp, _vp]),
     "fbfc_fft1d": (_i, [_vp, _l, _i, _i, _i, _vp, _vp]),
     "fbfc_ifft1d": (_i, [_vp, _l, _i, _i, _i, _vp, _vp]),
     "fbfc_transpose_mm": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _vp]),

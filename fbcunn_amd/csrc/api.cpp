@@ -632,10 +632,9 @@ int fbfc_backward(fbfc_plan *p, const float *input, const float *grad_output, co
     return acc_grad_parameters(p, input, grad_output, grad_weight, grad_bias, scale, true, stream);
 }
 
-int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
-               float *freq, void *stream)
+static int fft2d_impl(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
+                      float *freq, void *stream)
 {
-    fbfc::kernel_log_clear();
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
         return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
@@ -653,10 +652,16 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
     return FBFC_OK;
 }
 
-int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
-                float *real, const float *bias, int bias_period, void *stream)
+int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
+               float *freq, void *stream)
 {
     fbfc::kernel_log_clear();
+    return fft2d_impl(real, planes, h, w, pad_u, pad_l, fft_size, freq, stream);
+}
+
+static int ifft2d_impl(const float *freq, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
+                       float *real, const float *bias, int bias_period, void *stream)
+{
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
         return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
@@ -672,6 +677,82 @@ int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad
     }
     FBFC_TRY(fbfc::launch_irfft2d(fft_size, freq, real, planes, h, w, pad_u, pad_l, bias, bias_period,
                                   static_cast<hipStream_t>(stream)), "irfft2d");
+    return FBFC_OK;
+}
+
+int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
+                float *real, const float *bias, int bias_period, void *stream)
+{
+    fbfc::kernel_log_clear();
+    return ifft2d_impl(freq, planes, h, w, pad_u, pad_l, fft_size, real, bias, bias_period, stream);
+}
+
+// fbfft leaves a 2-D spectrum as (planes, N/2+1, N): rows = the halved axis.  Which axis that is
+// depends on the size (test/test_FFTModule.lua:238-241): see layout_kernels.hip.
+static int planes_layout_mode(int n) { return (n < 8 || n > 32) ? 1 : 2; }
+
+size_t fbfc_planes_layout_workspace_bytes(long planes, int fft_size)
+{
+    if (planes < 1 || (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))) return 0;
+    return (size_t)planes * fft_size * (fft_size / 2 + 1) * 8;
+}
+
+int fbfc_fft2d_planes(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
+                      float *freq_planes, float *workspace, void *stream)
+{
+    if (freq_planes == nullptr || workspace == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    fbfc::kernel_log_clear();
+    const int rc = fft2d_impl(real, planes, h, w, pad_u, pad_l, fft_size, workspace, stream);
+    if (rc != FBFC_OK) return rc;
+    FBFC_TRY(fbfc::launch_freq_to_planes(workspace, freq_planes, planes, fft_size * (fft_size / 2 + 1), fft_size,
+                                         planes_layout_mode(fft_size), static_cast<hipStream_t>(stream)),
+             "layout conversion");
+    return FBFC_OK;
+}
+
+int fbfc_ifft2d_planes(const float *freq_planes, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
+                       float *real, float *workspace, void *stream)
+{
+    if (freq_planes == nullptr || workspace == nullptr || real == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
+        return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
+    if (planes < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    fbfc::kernel_log_clear();
+    FBFC_TRY(fbfc::launch_planes_to_freq(freq_planes, workspace, planes, fft_size * (fft_size / 2 + 1), fft_size,
+                                         planes_layout_mode(fft_size), static_cast<hipStream_t>(stream)),
+             "layout conversion");
+    return ifft2d_impl(workspace, planes, h, w, pad_u, pad_l, fft_size, real, nullptr, 1, stream);
+}
+
+static int transpose_mm_impl(const float *A, const float *B, float *C, int n_freq, int m, int n, int k,
+                             float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate, void *stream);
+
+size_t fbfc_transpose_mm_planes_workspace_bytes(int n_freq, int m, int n, int k)
+{
+    if (n_freq < 1 || m < 1 || n < 1 || k < 1) return 0;
+    return (size_t)n_freq * 8 * ((size_t)m * k + (size_t)k * n + (size_t)m * n);
+}
+
+int fbfc_transpose_mm_planes(const float *A, const float *B, float *C, int n_freq, int m, int n, int k,
+                             float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate,
+                             float *workspace, void *stream)
+{
+    if (A == nullptr || B == nullptr || C == nullptr || workspace == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (n_freq < 1 || m < 1 || n < 1 || k < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    float *wa = workspace;
+    float *wb = wa + (size_t)n_freq * m * k * 2;
+    float *wc = wb + (size_t)n_freq * k * n * 2;
+    fbfc::kernel_log_clear();
+    FBFC_TRY(fbfc::launch_planes_to_freq(A, wa, (long)m * k, n_freq, 0, 0, s), "layout conversion (A)");
+    FBFC_TRY(fbfc::launch_planes_to_freq(B, wb, (long)k * n, n_freq, 0, 0, s), "layout conversion (B)");
+    if (accumulate) FBFC_TRY(fbfc::launch_planes_to_freq(C, wc, (long)m * n, n_freq, 0, 0, s), "layout conversion (C)");
+    const int rc = transpose_mm_impl(wa, wb, wc, n_freq, m, n, k, inv_norm, conj_trans_a, conj_trans_b, accumulate,
+                                     stream);
+    if (rc != FBFC_OK) return rc;
+    FBFC_TRY(fbfc::launch_freq_to_planes(wc, C, (long)m * n, n_freq, 0, 0, s), "layout conversion (C)");
     return FBFC_OK;
 }
 
@@ -701,10 +782,9 @@ int fbfc_ifft1d(const float *freq, long rows, int n, int pad_l, int fft_size, fl
     return FBFC_OK;
 }
 
-int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq, int m, int n, int k,
-                      float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate, void *stream)
+static int transpose_mm_impl(const float *A, const float *B, float *C, int n_freq, int m, int n, int k,
+                             float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate, void *stream)
 {
-    fbfc::kernel_log_clear();
     if (A == nullptr || B == nullptr || C == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (n_freq < 1 || m < 1 || n < 1 || k < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
     if (conj_trans_a && conj_trans_b)
@@ -713,6 +793,13 @@ int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq, int 
     FBFC_TRY(fbfc::launch_cgemm_freq(mode, A, B, C, n_freq, m, n, k, inv_norm, accumulate ? 1 : 0,
                                      static_cast<hipStream_t>(stream)), "cgemm");
     return FBFC_OK;
+}
+
+int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq, int m, int n, int k,
+                      float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate, void *stream)
+{
+    fbfc::kernel_log_clear();
+    return transpose_mm_impl(A, B, C, n_freq, m, n, k, inv_norm, conj_trans_a, conj_trans_b, accumulate, stream);
 }
 
 int fbfc_update_output_bias(float *output, const float *bias, int batch, int planes, int h, int w,

@@ -112,6 +112,14 @@ const char *kernel_log_get();
 // waves per block (falls back to the shape rule where the forced variant cannot run the shape).
 void cgemm_force_variant(int v);
 
+// layout_kernels.hip: frequency-major freq[q][plane] <-> the reference's plane-major buf[plane][q].
+// mode 0: same frequency order; 1: buf[a][c] = X[ky = c][kx = a] (fbfft for N < 8 or N > 32);
+// 2: buf[a][c] = X[ky = a][kx = c], a <= N/2 (fbfft for 8 <= N <= 32).  nq = entries per plane.
+hipError_t launch_freq_to_planes(const float *freq, float *buf, long planes, int nq, int N, int mode,
+                                 hipStream_t s);
+hipError_t launch_planes_to_freq(const float *buf, float *freq, long planes, int nq, int N, int mode,
+                                 hipStream_t s);
+
 // bias_kernels.hip ---------------------------------------------------------------
 hipError_t launch_bias_add(float *out, const float *bias, int batch, int planes, int hw,
                            hipStream_t s);

@@ -288,12 +288,38 @@ class FFTWrapper:
     every call is measured (1 skipped + 1 timed run, src/fft/FFTWrapperLua.cpp:106-134) and
     `lastTiming` holds {"ms", "GNlogN/s"} computed like the reference's log line (:137-152)."""
 
-    def __init__(self, cufft=None, padLeft=0, padUp=0, timed=False):
+    def __init__(self, cufft=None, padLeft=0, padUp=0, timed=False, layout="frequency"):
         if cufft not in (None, "fbfft", False, 0):
             raise ValueError("only the fbfft implementation exists in this build")
+        if layout not in ("frequency", "planes"):
+            raise ValueError("layout must be 'frequency' or 'planes'")
         self.padLeft, self.padUp = padLeft, padUp
         self.timed = bool(timed)
         self.lastTiming = None
+        # "planes": the reference's own 2-D buffer, (planes..., N/2+1, N, 2), first frequency axis
+        # halved and laid out as fbfft leaves it (test/test_FFTModule.lua:238-241)
+        self.layout = layout
+        self._workspace = None
+
+    def _planes_workspace(self, planes, n, device):
+        nbytes = lib().fbfc_planes_layout_workspace_bytes(planes, n)
+        if self._workspace is None or self._workspace.numel() * 4 < nbytes or self._workspace.device != device:
+            self._workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=device)
+        return self._workspace
+
+    def _dims_planes(self, time, frequency):
+        _check_tensor(time, "time")
+        _check_tensor(frequency, "frequency")
+        if frequency.dim() < 4 or frequency.size(-1) != 2:
+            raise ValueError("frequency must be (planes..., N/2+1, N, 2)")
+        n = frequency.size(-2)
+        if frequency.size(-3) != n // 2 + 1:
+            raise ValueError("frequency must be (planes..., N/2+1, N, 2)")
+        planes = frequency.numel() // (2 * n * (n // 2 + 1))
+        h, w = time.size(-2), time.size(-1)
+        if time.numel() != planes * h * w:
+            raise ValueError("time and frequency disagree on the number of planes")
+        return n, planes, h, w
 
     @staticmethod
     def _dims(time, frequency):
@@ -337,6 +363,12 @@ class FFTWrapper:
         self.lastTiming = {"ms": ms, "GNlogN/s": size / 1e9 / (ms * 1e-3) if ms > 0 else float("inf")}
 
     def fft(self, time, frequency, batchDims=None):
+        if self.layout == "planes" and frequency.dim() >= 4:
+            n, planes, h, w = self._dims_planes(time, frequency)
+            ws = self._planes_workspace(planes, n, time.device)
+            self._run(lambda: check(lib().fbfc_fft2d_planes(_ptr(time), planes, h, w, self.padUp, self.padLeft, n,
+                                                            _ptr(frequency), _ptr(ws), _stream())), 2, n, planes)
+            return frequency
         dims, n, planes, h, w = self._dims(time, frequency)
         if dims == 1:
             self._run(lambda: check(lib().fbfc_fft1d(_ptr(time), planes, w, self.padLeft, n, _ptr(frequency),
@@ -347,6 +379,14 @@ class FFTWrapper:
         return frequency
 
     def ffti(self, time, frequency, batchDims=None, bias=None):
+        if self.layout == "planes" and frequency.dim() >= 4:
+            if bias is not None:
+                raise ValueError("the plane-major inverse adds no bias")
+            n, planes, h, w = self._dims_planes(time, frequency)
+            ws = self._planes_workspace(planes, n, time.device)
+            self._run(lambda: check(lib().fbfc_ifft2d_planes(_ptr(frequency), planes, h, w, self.padUp, self.padLeft,
+                                                             n, _ptr(time), _ptr(ws), _stream())), 2, n, planes)
+            return time
         dims, n, planes, h, w = self._dims(time, frequency)
         if dims == 1:
             self._run(lambda: check(lib().fbfc_ifft1d(_ptr(frequency), planes, w, self.padLeft, n, _ptr(time),
@@ -358,8 +398,26 @@ class FFTWrapper:
         return time
 
 
-def transposeMM(A, B, C, invNorm, conjugateTransposeA, conjugateTransposeB, accumulate):
-    """transposeMMFFI (src/MM.cu:54-73) on frequency-major operands (Q, rows, cols, 2)."""
+def transposeMM(A, B, C, invNorm, conjugateTransposeA, conjugateTransposeB, accumulate, layout="frequency"):
+    """transposeMMFFI (src/MM.cu:54-73).  layout "frequency": operands (Q, rows, cols, 2);
+    layout "planes": the reference's own (rows, cols, f1, f2, 2) buffers, Q = f1 * f2."""
+    if layout == "planes":
+        for t, nme in ((A, "A"), (B, "B"), (C, "C")):
+            _check_tensor(t, nme, 5)
+        m, n = C.size(0), C.size(1)
+        Q = C.size(2) * C.size(3)
+        k = A.size(0) if conjugateTransposeA else A.size(1)
+        exp_a = (k, m) if conjugateTransposeA else (m, k)
+        exp_b = (n, k) if conjugateTransposeB else (k, n)
+        if tuple(A.shape[:2]) != exp_a or tuple(B.shape[:2]) != exp_b or \
+                tuple(A.shape[2:]) != tuple(C.shape[2:]) or tuple(B.shape[2:]) != tuple(C.shape[2:]):
+            raise ValueError("operand shapes do not match: A %s B %s C %s" % (tuple(A.shape), tuple(B.shape), tuple(C.shape)))
+        nbytes = lib().fbfc_transpose_mm_planes_workspace_bytes(Q, m, n, k)
+        ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=C.device)
+        check(lib().fbfc_transpose_mm_planes(_ptr(A), _ptr(B), _ptr(C), Q, m, n, k, ctypes.c_float(invNorm),
+                                             int(bool(conjugateTransposeA)), int(bool(conjugateTransposeB)),
+                                             int(bool(accumulate)), _ptr(ws), _stream()))
+        return C
     for t, nme in ((A, "A"), (B, "B"), (C, "C")):
         _check_tensor(t, nme, 4)
     Q, m, n = C.size(0), C.size(1), C.size(2)

@@ -179,7 +179,8 @@ int fbfc_debug_force_contraction_kernel(int variant);
  * fbfft2dHost, src/fft/FBFFTHost.cpp:39-116): batched 2-D real-to-complex FFT of
  * `planes` h x w planes, each implicitly zero-padded into an N x N canvas at
  * row pad_u, column pad_l.  N in {2,4,8,16,32,64,128} (the sizes the reference tests,
- * test/test_FFTModule.lua:170-260).  Output is frequency-major. */
+ * test/test_FFTModule.lua:170-260).  Output is frequency-major (fbfc_fft2d_planes gives the
+ * reference's plane-major buffer). */
 int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l,
                int fft_size, float *freq, void *stream);
 
@@ -192,6 +193,20 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
  * conjugates of (N - ky, kx). */
 int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l,
                 int fft_size, float *real, const float *bias, int bias_period, void *stream);
+
+/* The same two transforms on the reference's own buffer layout, for callers at the nn.FFTWrapper
+ * level (fbcunn/FFTWrapper.lua:53-132, test/test_FFTModule.lua:238-342): freq_planes is
+ * (planes, N/2+1, N, 2), plane-major, the first of the two frequency axes halved.  As fbfft leaves
+ * it, buf[a][c] = X[ky = a][kx = c] for 8 <= N <= 32 and buf[a][c] = X[ky = c][kx = a] for N < 8 or
+ * N > 32 (test/test_FFTModule.lua:238-241).  workspace: fbfc_planes_layout_workspace_bytes(planes, N)
+ * bytes of device memory, the counterpart of the buffer tensor the reference passes for sizes above
+ * 32 (fbcunn/FFTWrapper.lua:73-79, 114-122); the transform runs frequency-major in it and one more
+ * kernel converts the layout.  The inverse is unnormalised and reads the whole half plane given. */
+size_t fbfc_planes_layout_workspace_bytes(long planes, int fft_size);
+int fbfc_fft2d_planes(const float *real, long planes, int h, int w, int pad_u, int pad_l,
+                      int fft_size, float *freq_planes, float *workspace, void *stream);
+int fbfc_ifft2d_planes(const float *freq_planes, long planes, int h, int w, int pad_u, int pad_l,
+                       int fft_size, float *real, float *workspace, void *stream);
 
 /* Replaces FFTWrapper_fft / FFTWrapper_ffti on tensors with ONE transform dimension
  * (fbfft1dHost, src/fft/FBFFTHost.cpp:119-131): `rows` real sequences of n values, each
@@ -210,6 +225,16 @@ int fbfc_ifft1d(const float *freq, long rows, int n, int pad_l, int fft_size, fl
 int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq,
                       int m, int n, int k, float inv_norm,
                       int conj_trans_a, int conj_trans_b, int accumulate, void *stream);
+
+/* transposeMMFFI on the reference's operand layout (src/MM.cu:14-24, 54-73): A, B, C are
+ * (rows, cols, n_freq, 2), plane-major, as the (d0, d1, N/2+1, N, 2) buffers of
+ * fbcunn/SpatialConvolutionFFT.lua:710-721 are with their two frequency axes flattened.  Same
+ * arithmetic as fbfc_transpose_mm; the operands are brought to frequency-major order in `workspace`
+ * (fbfc_transpose_mm_planes_workspace_bytes bytes) and C is written back plane-major. */
+size_t fbfc_transpose_mm_planes_workspace_bytes(int n_freq, int m, int n, int k);
+int fbfc_transpose_mm_planes(const float *A, const float *B, float *C, int n_freq,
+                             int m, int n, int k, float inv_norm, int conj_trans_a, int conj_trans_b,
+                             int accumulate, float *workspace, void *stream);
 
 /* Replaces updateOutputBiasFFI (src/ConvolutionBias.cu:256-260): output[b][f][.][.] += bias[f]. */
 int fbfc_update_output_bias(float *output, const float *bias, int batch, int planes,

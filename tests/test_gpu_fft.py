@@ -232,3 +232,67 @@ def test_plane_count_beyond_the_32_bit_row_offsets_is_refused(nn):
                            ctypes.c_void_p(small.data_ptr()), ctypes.c_void_p(0), 1, ctypes.c_void_p(0))
     assert rc != 0
     torch.cuda.synchronize()
+
+
+# ---- the reference's own buffer layout (nn.FFTWrapper level) -------------------------------------
+def _reference_layout(full, n):
+    """complex (planes, N, N) full spectrum X[ky][kx] -> the (planes, N/2+1, N) buffer fbfft leaves:
+    buf[a][c] = X[ky = a][kx = c] for 8 <= N <= 32, buf[a][c] = X[ky = c][kx = a] otherwise
+    (test/test_FFTModule.lua:238-241, 267-269)."""
+    if 8 <= n <= 32:
+        return full[:, :n // 2 + 1, :]
+    return np.transpose(full, (0, 2, 1))[:, :n // 2 + 1, :]
+
+
+PLANES_CASES = [(4, 7, 3, 2, 1, 2), (8, 33, 5, 6, 2, 1), (16, 200, 13, 13, 1, 1), (32, 70, 27, 27, 2, 2),
+                (32, 48, 32, 32, 0, 0), (64, 37, 55, 55, 4, 4), (64, 41, 9, 9, 0, 0), (128, 5, 100, 100, 3, 7)]
+
+
+@pytest.mark.parametrize("n,planes,h,w,pu,pl", PLANES_CASES)
+def test_forward_in_the_reference_layout(nn, oracle, n, planes, h, w, pu, pl):
+    x = synth.uniform(300 + n, (planes, h, w))
+    freq = torch.full((planes, n // 2 + 1, n, 2), float("nan"), device="cuda")
+    nn.FFTWrapper("fbfft", pl, pu, layout="planes").fft(dev(x), freq)
+    got = host(freq)
+    got = got[..., 0] + 1j * got[..., 1]
+    full = np.fft.fft2(_canvas(x, n, pu, pl))
+    want = _reference_layout(full, n)
+    scale = np.abs(want).max()
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL * scale
+    # the oracle's naive DFT gives X[ky][kx <= N/2]; the other half follows from X[-ky][-kx] = conj X[ky][kx]
+    pick = sorted({0, planes - 1})
+    o = oracle.dft2d_r2c(x[pick], n, n, pu, pl)
+    half = o[..., 0] + 1j * o[..., 1]                       # (len(pick), N, N/2+1)
+    fullo = np.zeros((len(pick), n, n), complex)
+    fullo[:, :, :n // 2 + 1] = half
+    for kx in range(n // 2 + 1, n):
+        fullo[:, :, kx] = np.conj(half[:, (-np.arange(n)) % n, n - kx])
+    assert np.abs(got[pick] - _reference_layout(fullo, n)).max() <= TOL * scale
+
+
+@pytest.mark.parametrize("n,planes,h,w,pu,pl", PLANES_CASES)
+def test_inverse_in_the_reference_layout(nn, n, planes, h, w, pu, pl):
+    full = synth.uniform(400 + n, (planes, n, n))
+    spec = _reference_layout(np.fft.fft2(full.astype(np.float64)), n)
+    buf = dev(np.stack([spec.real, spec.imag], -1).astype(np.float32))
+    out = torch.full((planes, h, w), float("nan"), device="cuda")
+    nn.FFTWrapper("fbfft", pl, pu, layout="planes").ffti(out, buf)
+    want = full[:, pu:pu + h, pl:pl + w].astype(np.float64) * (n * n)
+    got = host(out)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= TOL * np.abs(want).max() * 4
+
+
+def test_round_trip_in_the_reference_layout(nn):
+    """fft then ffti / N^2 on (batch, planes, N, N) tensors with two batch dimensions, as
+    test/test_FFTModule.lua:247-262 runs it."""
+    n = 32
+    x = synth.uniform(55, (3, 5, n, n))
+    xd = dev(x)
+    freq = torch.empty((3, 5, n // 2 + 1, n, 2), device="cuda")
+    w = nn.FFTWrapper("fbfft", layout="planes")
+    w.fft(xd, freq, 2)
+    back = torch.empty_like(xd)
+    w.ffti(back, freq, 2)
+    assert np.abs(host(back) / (n * n) - x).max() <= 1e-5 * np.abs(x).max()

@@ -98,3 +98,29 @@ def test_both_conjugations_rejected(nn):
     with pytest.raises(nn.FbfcError) as e:
         nn.transposeMM(t, t, t.clone(), 1.0, True, True, False)
     assert e.value.code == 3
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_transpose_mm_on_the_reference_operand_layout(nn, mode):
+    """src/MM.cu:14-24, 54-73: operands are (d0, d1, N/2+1, N, 2) buffers, plane-major."""
+    f1, f2, m, n, k = 9, 16, 20, 12, 7
+    rng = np.random.RandomState(5 + mode)
+    cplx = lambda *shape: rng.uniform(-1, 1, shape) + 1j * rng.uniform(-1, 1, shape)
+    conj_a, conj_b = mode == 2, mode == 0
+    A = cplx(k, m, f1, f2) if conj_a else cplx(m, k, f1, f2)
+    B = cplx(n, k, f1, f2) if conj_b else cplx(k, n, f1, f2)
+    C0 = cplx(m, n, f1, f2)
+    if mode == 0:
+        want = np.einsum("mkxy,nkxy->mnxy", A, np.conj(B))
+    elif mode == 1:
+        want = np.einsum("mkxy,knxy->mnxy", A, B)
+    else:
+        want = np.einsum("kmxy,knxy->mnxy", np.conj(A), B)
+    pack = lambda z: dev(np.stack([z.real, z.imag], -1).astype(np.float32))
+    for accumulate in (False, True):
+        Cd = pack(C0)
+        nn.transposeMM(pack(A), pack(B), Cd, 0.5, conj_a, conj_b, accumulate, layout="planes")
+        got = host(Cd)
+        got = got[..., 0] + 1j * got[..., 1]
+        exp = 0.5 * want + (C0 if accumulate else 0)
+        assert np.abs(got - exp).max() <= 2e-5 * np.abs(exp).max()
