@@ -71,6 +71,9 @@ SIGNATURES = {
     "fbfc_fft1d": (_i, [_vp, _l, _i, _i, _i, _vp, _vp]),
     "fbfc_ifft1d": (_i, [_vp, _l, _i, _i, _i, _vp, _vp]),
     "fbfc_transpose_mm": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _vp]),
+    "fbfc_direct_update_output": (_i, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp]),
+    "fbfc_direct_update_grad_input": (_i, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp]),
+    "fbfc_direct_acc_grad_parameters": (_i, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _f, _vp, _vp]),
     "fbfc_update_output_bias": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "fbfc_update_output_bias_strided": (_i, [_vp, _vp, _i, _i, _i, _i, _l, _l, _l, _l, _l, _vp]),
     "fbfc_acc_grad_parameters_bias_strided": (_i, [_vp, _vp, _f, _i, _i, _i, _i, _l, _l, _l, _l, _l, _vp, _vp]),

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libfbfftconv.so")
-SOURCES = ["api.cpp", "fft_kernels.hip", "fft_large.hip", "fft_small.hip", "cgemm_kernels.hip", "bias_kernels.hip", "bias_noalloc.hip", "layout_kernels.hip"]
+SOURCES = ["api.cpp", "fft_kernels.hip", "fft_large.hip", "fft_small.hip", "cgemm_kernels.hip", "bias_kernels.hip", "bias_noalloc.hip", "layout_kernels.hip", "direct_kernels.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",

@@ -802,6 +802,69 @@ int fbfc_transpose_mm(const float *A, const float *B, float *C, int n_freq, int 
     return transpose_mm_impl(A, B, C, n_freq, m, n, k, inv_norm, conj_trans_a, conj_trans_b, accumulate, stream);
 }
 
+// ---- direct convolution -------------------------------------------------------------------------
+static int direct_check(const fbfc_conv_desc *d)
+{
+    if (d == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (d->batch < 1 || d->in_planes < 1 || d->out_planes < 1 || d->in_h < 1 || d->in_w < 1 || d->k_h < 1 ||
+        d->k_w < 1 || d->stride_h < 1 || d->stride_w < 1)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    if (d->pad_h < 0 || d->pad_w < 0) return fail(FBFC_ERR_INVALID_ARGUMENT, "padding must be non-negative");
+    if (d->in_h + 2 * d->pad_h < d->k_h || d->in_w + 2 * d->pad_w < d->k_w)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "kernel larger than padded input");
+    return FBFC_OK;
+}
+
+static_assert(sizeof(fbfc_conv_desc) == 11 * sizeof(int), "the direct kernels read the descriptor as 11 ints");
+
+int fbfc_direct_update_output(const fbfc_conv_desc *desc, const float *input, const float *weight,
+                              const float *bias, float *output, void *stream)
+{
+    const int rc = direct_check(desc);
+    if (rc != FBFC_OK) return rc;
+    if (input == nullptr || weight == nullptr || output == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    fbfc::kernel_log_clear();
+    FBFC_TRY(fbfc::launch_direct_fprop(reinterpret_cast<const int *>(desc), input, weight, bias, output,
+                                       static_cast<hipStream_t>(stream)), "direct updateOutput");
+    return FBFC_OK;
+}
+
+int fbfc_direct_update_grad_input(const fbfc_conv_desc *desc, const float *grad_output, const float *weight,
+                                  float *grad_input, void *stream)
+{
+    const int rc = direct_check(desc);
+    if (rc != FBFC_OK) return rc;
+    if (grad_output == nullptr || weight == nullptr || grad_input == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    fbfc::kernel_log_clear();
+    FBFC_TRY(fbfc::launch_direct_bprop(reinterpret_cast<const int *>(desc), grad_output, weight, grad_input,
+                                       static_cast<hipStream_t>(stream)), "direct updateGradInput");
+    return FBFC_OK;
+}
+
+int fbfc_direct_acc_grad_parameters(const fbfc_conv_desc *desc, const float *input, const float *grad_output,
+                                    float *grad_weight, float *grad_bias, float scale, float *scratch,
+                                    void *stream)
+{
+    const int rc = direct_check(desc);
+    if (rc != FBFC_OK) return rc;
+    if (input == nullptr || grad_output == nullptr || grad_weight == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (grad_bias != nullptr && scratch == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "the bias gradient needs its workspace");
+    fbfc::kernel_log_clear();
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    FBFC_TRY(fbfc::launch_direct_accgrad(reinterpret_cast<const int *>(desc), input, grad_output, grad_weight, scale,
+                                         s), "direct accGradParameters");
+    if (grad_bias != nullptr) {
+        const int o_h = (desc->in_h + 2 * desc->pad_h - desc->k_h) / desc->stride_h + 1;
+        const int o_w = (desc->in_w + 2 * desc->pad_w - desc->k_w) / desc->stride_w + 1;
+        FBFC_TRY(fbfc::launch_bias_grad(grad_output, grad_bias, scale, desc->batch, desc->out_planes, o_h * o_w,
+                                        scratch, s), "bias grad");
+    }
+    return FBFC_OK;
+}
+
 int fbfc_update_output_bias(float *output, const float *bias, int batch, int planes, int h, int w,
                             void *stream)
 {

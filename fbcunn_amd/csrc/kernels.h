@@ -120,6 +120,13 @@ hipError_t launch_freq_to_planes(const float *freq, float *buf, long planes, int
 hipError_t launch_planes_to_freq(const float *buf, float *freq, long planes, int nq, int N, int mode,
                                  hipStream_t s);
 
+// direct_kernels.hip: spatial-domain convolution (any stride).  desc = the 11 ints of fbfc_conv_desc.
+hipError_t launch_direct_fprop(const int *desc, const float *in, const float *w, const float *bias, float *out,
+                               hipStream_t s);
+hipError_t launch_direct_bprop(const int *desc, const float *go, const float *w, float *gi, hipStream_t s);
+hipError_t launch_direct_accgrad(const int *desc, const float *in, const float *go, float *gw, float scale,
+                                 hipStream_t s);
+
 // bias_kernels.hip ---------------------------------------------------------------
 hipError_t launch_bias_add(float *out, const float *bias, int batch, int planes, int hw,
                            hipStream_t s);

@@ -15,7 +15,7 @@ import torch
 from . import _lib
 from ._lib import ConvDesc, FbfcError, PlanInfo, check, lib
 
-__all__ = ["SpatialConvolutionFFT", "SpatialConvolutionFBFFT", "SpatialConvolutionFBFFTGemm",
+__all__ = ["SpatialConvolutionFFT", "SpatialConvolutionFBFFT", "SpatialConvolutionFBFFTGemm", "SpatialConvolutionDirect",
            "SpatialConvolutionFFTTiled", "SpatialConvolutionFFTTiledSync", "SpatialConvolutionFFTTiledAsync",
            "SpatialConvolutionFFTTiledIterated", "FFTWrapper", "transposeMM", "updateOutputBias", "accGradParametersBias", "FbfcError"]
 
@@ -63,9 +63,86 @@ class _Plan:
             pass
 
 
+class SpatialConvolutionDirect:
+    """The direct (spatial-domain) convolution, in the role cudnn.SpatialConvolution plays next to the
+    reference's FFT modules: non-FFT candidate of the tuning front (fbcunn/SpatialConvolution.lua:259-269),
+    fallback for layers the FFT path cannot run (fbcunn/SpatialConvolutionFFT.lua:323-393) and the
+    result the self-check compares with (:91-133).  Any stride.  accGradParameters assigns gradWeight
+    and gradBias, like the FFT modules here."""
+
+    def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padW=0, padH=0, device="cuda"):
+        self.nInputPlane, self.nOutputPlane = nInputPlane, nOutputPlane
+        self.kW, self.kH, self.dW, self.dH, self.padW, self.padH = kW, kH, dW, dH, padW, padH
+        self.device = torch.device(device)
+        self.weight = torch.empty(nOutputPlane, nInputPlane, kH, kW, device=self.device)
+        self.bias = torch.empty(nOutputPlane, device=self.device)
+        self.gradWeight = torch.zeros(nOutputPlane, nInputPlane, kH, kW, device=self.device)
+        self.gradBias = torch.zeros(nOutputPlane, device=self.device)
+        self.output = None
+        self.gradInput = None
+        stdv = 1.0 / math.sqrt(kW * kH * nInputPlane)
+        self.weight.uniform_(-stdv, stdv)
+        self.bias.uniform_(-stdv, stdv)
+
+    def _desc(self, input):
+        _check_tensor(input, "input", 4)
+        if input.size(1) != self.nInputPlane:
+            raise ValueError("input has %d planes, module expects %d" % (input.size(1), self.nInputPlane))
+        return ConvDesc(input.size(0), self.nInputPlane, self.nOutputPlane, input.size(2), input.size(3),
+                        self.kH, self.kW, self.dH, self.dW, self.padH, self.padW)
+
+    def _out_shape(self, input):
+        return (input.size(0), self.nOutputPlane, (input.size(2) + 2 * self.padH - self.kH) // self.dH + 1,
+                (input.size(3) + 2 * self.padW - self.kW) // self.dW + 1)
+
+    def updateOutput(self, input):
+        d = self._desc(input)
+        shape = self._out_shape(input)
+        if self.output is None or tuple(self.output.shape) != shape:
+            self.output = torch.empty(shape, device=input.device)
+        check(lib().fbfc_direct_update_output(ctypes.byref(d), _ptr(input), _ptr(self.weight), _ptr(self.bias),
+                                              _ptr(self.output), _stream()))
+        return self.output
+
+    forward = updateOutput
+
+    def updateGradInput(self, input, gradOutput):
+        d = self._desc(input)
+        _check_tensor(gradOutput, "gradOutput", 4)
+        if tuple(gradOutput.shape) != self._out_shape(input):
+            raise ValueError("gradOutput has the wrong shape")
+        if self.gradInput is None or self.gradInput.shape != input.shape:
+            self.gradInput = torch.empty_like(input)
+        check(lib().fbfc_direct_update_grad_input(ctypes.byref(d), _ptr(gradOutput), _ptr(self.weight),
+                                                  _ptr(self.gradInput), _stream()))
+        return self.gradInput
+
+    def accGradParameters(self, input, gradOutput, scale=1.0):
+        d = self._desc(input)
+        _check_tensor(gradOutput, "gradOutput", 4)
+        if tuple(gradOutput.shape) != self._out_shape(input):
+            raise ValueError("gradOutput has the wrong shape")
+        nbytes = lib().fbfc_bias_grad_scratch_bytes(input.size(0), self.nOutputPlane)
+        scratch = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=input.device)
+        check(lib().fbfc_direct_acc_grad_parameters(ctypes.byref(d), _ptr(input), _ptr(gradOutput),
+                                                    _ptr(self.gradWeight), _ptr(self.gradBias),
+                                                    ctypes.c_float(scale), _ptr(scratch), _stream()))
+
+    def backward(self, input, gradOutput, scale=1.0):
+        self.updateGradInput(input, gradOutput)
+        self.accGradParameters(input, gradOutput, scale)
+        return self.gradInput
+
+    def cleanupBuffers(self):
+        pass
+
+
 class SpatialConvolutionFFT:
     """Module state and protocol of nn.SpatialConvolutionFFT
     (fbcunn/SpatialConvolutionFFT.lua:150-316, 405-416)."""
+
+    # relative-L2 bound of the self-check (fbcunn/SpatialConvolutionFFT.lua:15)
+    prec = 2e-5
 
     memoryReuseNone = "none"
     memoryReuseInput = "input"
@@ -108,8 +185,31 @@ class SpatialConvolutionFFT:
         self.output = None
         self.gradInput = None
         self.timed = False
+        # the reference's debugging hook (fbcunn/SpatialConvolutionFFT.lua:160-161, 91-133): with
+        # cudnnDebug set every pass is run again through the direct convolution and cudnnChecks turns
+        # False when they differ by more than `prec` in relative L2
+        self.cudnnDebug = False
+        self.cudnnChecks = True
+        self.printDebugLevel = -1
         self._plans = {}
         self.reset()
+
+    def debugVSCUDNN(self, pass_name, got, run_direct):
+        """Compares `got` with what the direct path computes for the same pass (run_direct(module) ->
+        tensor); ||direct - got|| / ||direct|| must not exceed self.prec."""
+        other = SpatialConvolutionDirect(self.nInputPlane, self.nOutputPlane, self.kW, self.kH, self.dW, self.dH,
+                                         self.padLeft, self.padUp, device=self.device)
+        other.weight, other.bias = self.weight, self.bias
+        want = run_direct(other).double()
+        norm = math.sqrt(float(torch.dot(want.flatten(), want.flatten())) + 1e-8)
+        err = float((want - got.double()).norm()) / norm
+        ok = bool(torch.isfinite(got).all()) and err <= self.prec
+        if not ok:
+            print("%s error %s %g %g" % (type(self).__name__, pass_name, err, self.prec))
+        elif self.printDebugLevel >= 0:
+            print("%s debug vs direct check passes %s %g" % (type(self).__name__, pass_name, err))
+        self.cudnnChecks = self.cudnnChecks and ok
+        return ok
 
     # -- parameters ---------------------------------------------------------------
     def reset(self, stdv=None):
@@ -181,6 +281,8 @@ class SpatialConvolutionFFT:
             self.output = torch.empty(shape, device=input.device)
         check(lib().fbfc_update_output(plan.handle, _ptr(input), _ptr(self.weight), _ptr(self.bias),
                                        _ptr(self.output), _stream()))
+        if self.cudnnDebug:
+            self.debugVSCUDNN("updateOutput", self.output, lambda m: m.updateOutput(input))
         return self.output
 
     forward = updateOutput
@@ -196,6 +298,8 @@ class SpatialConvolutionFFT:
             self.gradInput = torch.empty_like(input)
         check(lib().fbfc_update_grad_input(plan.handle, _ptr(gradOutput), _ptr(self.weight),
                                            _ptr(self.gradInput), _stream()))
+        if self.cudnnDebug:
+            self.debugVSCUDNN("updateGradInput", self.gradInput, lambda m: m.updateGradInput(input, gradOutput))
         return self.gradInput
 
     def accGradParameters(self, input, gradOutput, scale=1.0):
@@ -210,6 +314,11 @@ class SpatialConvolutionFFT:
         check(lib().fbfc_acc_grad_parameters(plan.handle, _ptr(input), _ptr(gradOutput),
                                              _ptr(self.gradWeight), _ptr(self.gradBias),
                                              ctypes.c_float(scale), _stream()))
+        if self.cudnnDebug:
+            def both(m):
+                m.accGradParameters(input, gradOutput, scale)
+                return torch.cat([m.gradWeight.flatten(), m.gradBias.flatten()])
+            self.debugVSCUDNN("accGradParameters", torch.cat([self.gradWeight.flatten(), self.gradBias.flatten()]), both)
 
     def backward(self, input, gradOutput, scale=1.0):
         """updateGradInput + accGradParameters sharing FFT(gradOutput)

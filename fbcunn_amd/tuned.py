@@ -1,8 +1,9 @@
 """Host-side mirror of fbnn.SpatialConvolution (fbcunn/SpatialConvolution.lua): the front
-that, on the first updateOutput, times the FFT strategies that fit the layer and keeps the
-fastest (:188-422).  The reference also times cuDNN and falls back to it; this build has
-no direct-convolution path, so the candidates are the FFT strategies only and a layer none
-of them can run (stride above 1, sizes out of range) raises.
+that, on the first updateOutput, times the strategies that fit the layer and keeps the
+fastest (:188-422).  Candidates: the FFT modules (untiled, tiles of 16 and 32, with and
+without memory reuse) and the direct convolution, which stands where the reference has
+cuDNN: it runs every layer (strides above 1, sizes no transform covers) and it is what
+the winner is checked against after tuning (:387-399), to the reference's 2e-5.
 """
 import time
 
@@ -42,11 +43,11 @@ class SpatialConvolution:
         self.inferenceOnly = bool(inferenceOnly)
         self.reportLevel = 0
         self.device = torch.device(device)
+        # after tuning, run the winning FFT strategy against the direct convolution (the reference
+        # always does, fbcunn/SpatialConvolution.lua:387-399) and fail if they differ
+        self.selfCheck = True
         # parameters live here and are handed to the strategy that wins
-        holder = nn.SpatialConvolutionFBFFT(nInputPlane, nOutputPlane, kW, kH, 1, 1, 0, 0, device=device) \
-            if (dW == 1 and dH == 1) else None
-        if holder is None:
-            raise ValueError("fft only supports stride-1 convolutions atm (and there is no direct path here)")
+        holder = nn.SpatialConvolutionDirect(nInputPlane, nOutputPlane, kW, kH, dW, dH, padLeft, padUp, device=device)
         self.weight, self.bias = holder.weight, holder.bias
         self.gradWeight, self.gradBias = holder.gradWeight, holder.gradBias
         self.output = None
@@ -61,7 +62,10 @@ class SpatialConvolution:
     # -- candidates (SpatialConvolution.lua:237-300) -----------------------------------
     def _candidates(self, iH, iW):
         reuse_all, reuse_none = nn.SpatialConvolutionFFT.memoryReuseAll, nn.SpatialConvolutionFFT.memoryReuseNone
-        cands = [("SpatialConvolutionFBFFT", None, reuse_all), ("SpatialConvolutionFBFFT", None, reuse_none)]
+        direct = ("SpatialConvolutionDirect", None, reuse_none)
+        if self.dW != 1 or self.dH != 1:
+            return [direct]         # "fft only supports stride-1 convolutions atm"
+        cands = [direct, ("SpatialConvolutionFBFFT", None, reuse_all), ("SpatialConvolutionFBFFT", None, reuse_none)]
         if self.kH <= 9 and self.kW <= 9:
             tiles = (16, 32)
         else:
@@ -85,7 +89,9 @@ class SpatialConvolution:
 
     def _make(self, cls, tile, reuse):
         args = (self.inputPlanes, self.outputPlanes, self.kW, self.kH, self.dW, self.dH, self.padLeft, self.padUp)
-        if tile is None:
+        if cls == "SpatialConvolutionDirect":
+            inst = nn.SpatialConvolutionDirect(*args, device=self.device)
+        elif tile is None:
             inst = getattr(nn, cls)(*args, reuse, device=self.device)
         else:
             inst = getattr(nn, cls)(*args, tile, tile, reuse, device=self.device)
@@ -95,15 +101,14 @@ class SpatialConvolution:
 
     def _tune(self, input):
         B, _, iH, iW = input.shape
-        oH = iH + 2 * self.padUp - self.kH + 1
-        oW = iW + 2 * self.padLeft - self.kW + 1
+        oH, oW = (iH + 2 * self.padUp - self.kH) // self.dH + 1, (iW + 2 * self.padLeft - self.kW) // self.dW + 1
         grad_output = torch.zeros(B, self.outputPlanes, max(oH, 1), max(oW, 1), device=input.device)
         # tuning must not disturb the caller's gradients
         keep_gw, keep_gb = self.gradWeight.clone(), self.gradBias.clone()
         best, best_ms = None, float("inf")
         self.timings = {}
         for cls, tile, reuse in self._candidates(iH, iW):
-            nbytes = self._plan_bytes(B, iH, iW, tile, reuse)
+            nbytes = 0 if cls == "SpatialConvolutionDirect" else self._plan_bytes(B, iH, iW, tile, reuse)
             key = (cls, tile, reuse)
             if nbytes is None:
                 self.timings[key] = None          # the strategy cannot run this layer
@@ -132,11 +137,23 @@ class SpatialConvolution:
                 self.bestKey = key
             else:
                 inst.cleanupBuffers()
+        if best is None:
+            raise _lib.FbfcError(_lib.ERR_UNSUPPORTED_SIZE, "no strategy can run this layer")
+        # correctness check of an FFT winner against the direct convolution, on random data
+        if self.selfCheck and not isinstance(best, nn.SpatialConvolutionDirect):
+            best.cudnnDebug, best.cudnnChecks = True, True
+            x = torch.randn_like(input)
+            g = torch.randn_like(grad_output)
+            best.updateOutput(x)
+            if not self.inferenceOnly:
+                best.updateGradInput(x, g)
+                best.accGradParameters(x, g, 1.0)
+            best.cudnnDebug = False
+            if not best.cudnnChecks:
+                best.cleanupBuffers()
+                raise _lib.FbfcError(_lib.ERR_HIP, "self-check of %s against the direct convolution failed" % (self.bestKey,))
         self.gradWeight.copy_(keep_gw)
         self.gradBias.copy_(keep_gb)
-        if best is None:
-            raise _lib.FbfcError(_lib.ERR_UNSUPPORTED_SIZE,
-                                 "no FFT strategy can run this layer (and there is no direct path here)")
         if self.reportLevel >= 1:
             print("Best FFT: ", best_ms, " ", self.bestKey)
         self.bestModuleInst = best

@@ -236,6 +236,21 @@ int fbfc_transpose_mm_planes(const float *A, const float *B, float *C, int n_fre
                              int m, int n, int k, float inv_norm, int conj_trans_a, int conj_trans_b,
                              int accumulate, float *workspace, void *stream);
 
+/* Direct (spatial-domain) convolution: the three passes for ANY stride and padding, without a plan.
+ * The role cudnn.SpatialConvolution plays for the reference's FFT path: the non-FFT candidate of the
+ * tuning front (fbcunn/SpatialConvolution.lua:259-269), the path a layer falls back to when the FFT
+ * modules cannot run it (fbcunn/SpatialConvolutionFFT.lua:323-393) and the result the self-check
+ * compares with (:91-133, :387-399).  Plain kernels, correct for every shape, not tuned.  Output size
+ * (in + 2 pad - k) / stride + 1; bias / grad_bias may be NULL; grad_weight and grad_bias are
+ * assigned; scratch: fbfc_bias_grad_scratch_bytes(batch, out_planes) bytes, needed with grad_bias. */
+int fbfc_direct_update_output(const fbfc_conv_desc *desc, const float *input, const float *weight,
+                              const float *bias, float *output, void *stream);
+int fbfc_direct_update_grad_input(const fbfc_conv_desc *desc, const float *grad_output,
+                                  const float *weight, float *grad_input, void *stream);
+int fbfc_direct_acc_grad_parameters(const fbfc_conv_desc *desc, const float *input,
+                                    const float *grad_output, float *grad_weight, float *grad_bias,
+                                    float scale, float *scratch, void *stream);
+
 /* Replaces updateOutputBiasFFI (src/ConvolutionBias.cu:256-260): output[b][f][.][.] += bias[f]. */
 int fbfc_update_output_bias(float *output, const float *bias, int batch, int planes,
                             int h, int w, void *stream);

@@ -58,6 +58,13 @@ size_t fbfc_transpose_mm_planes_workspace_bytes(int n_freq, int m, int n, int k)
 int fbfc_transpose_mm_planes(const float *A, const float *B, float *C, int n_freq, int m, int n, int k,
                              float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate,
                              float *workspace, void *stream);
+int fbfc_direct_update_output(const fbfc_conv_desc *desc, const float *input, const float *weight,
+                              const float *bias, float *output, void *stream);
+int fbfc_direct_update_grad_input(const fbfc_conv_desc *desc, const float *grad_output,
+                                  const float *weight, float *grad_input, void *stream);
+int fbfc_direct_acc_grad_parameters(const fbfc_conv_desc *desc, const float *input,
+                                    const float *grad_output, float *grad_weight, float *grad_bias,
+                                    float scale, float *scratch, void *stream);
 int fbfc_update_output_bias(float *output, const float *bias, int batch, int planes, int h, int w,
                             void *stream);
 int fbfc_update_output_bias_strided(float *output, const float *bias, int batch, int planes, int h, int w,
