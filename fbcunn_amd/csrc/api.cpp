@@ -199,6 +199,8 @@ struct fbfc_plan {
     pass_geom fprop, bprop, accgrad;
     int device;
     float *in_freq, *w_freq, *out_freq, *res_freq, *scratch;
+    float *bw_gi, *bw_gw;  // result spectra of fbfc_backward's single-grid stages, made at its first call
+    bool bw_failed;
     unsigned reuse;
     bool have_in, have_w, have_out;  // which forward spectra are valid in their buffer
     int timed;
@@ -405,6 +407,8 @@ int fbfc_plan_destroy(fbfc_plan *p)
     if (p->out_freq) (void)hipFree(p->out_freq);
     if (p->res_freq) (void)hipFree(p->res_freq);
     if (p->scratch) (void)hipFree(p->scratch);
+    if (p->bw_gi) (void)hipFree(p->bw_gi);
+    if (p->bw_gw) (void)hipFree(p->bw_gw);
     if (p->ev_made)
         for (hipEvent_t &ev : p->ev) (void)hipEventDestroy(ev);
     delete p;
@@ -622,14 +626,88 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
     return acc_grad_parameters(p, input, grad_output, grad_weight, grad_bias, scale, false, stream);
 }
 
+// The buffers the one-grid-per-stage backward pass writes its two product spectra to (it reads all
+// three operand spectra in one launch, so neither result may overwrite one of them).
+static bool backward_buffers(fbfc_plan *p)
+{
+    if (p->bw_gi != nullptr && p->bw_gw != nullptr) return true;
+    if (p->bw_failed) return false;
+    hipError_t e = hipSuccess;
+    if (p->bw_gi == nullptr) e = hipMalloc(reinterpret_cast<void **>(&p->bw_gi), p->info.input_freq_bytes);
+    if (e == hipSuccess && p->bw_gw == nullptr)
+        e = hipMalloc(reinterpret_cast<void **>(&p->bw_gw), p->info.weight_freq_bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        p->bw_failed = true;  // no room: the pass runs as its two halves, which need no extra buffer
+        return false;
+    }
+    return true;
+}
+
 int fbfc_backward(fbfc_plan *p, const float *input, const float *grad_output, const float *weight,
                   float *grad_input, float *grad_weight, float *grad_bias, float scale, void *stream)
 {
-    const int rc = fbfc_update_grad_input(p, grad_output, weight, grad_input, stream);
-    if (rc != FBFC_OK) return rc;
-    // updateGradInput leaves FFT(gradOutput) in the plan (have_out; not for tiled plans, whose two
-    // passes window gradOutput differently)
-    return acc_grad_parameters(p, input, grad_output, grad_weight, grad_bias, scale, true, stream);
+    if (p == nullptr || input == nullptr || grad_output == nullptr || weight == nullptr ||
+        grad_input == nullptr || grad_weight == nullptr)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (p->tiled || !backward_buffers(p)) {
+        const int rc = fbfc_update_grad_input(p, grad_output, weight, grad_input, stream);
+        if (rc != FBFC_OK) return rc;
+        // updateGradInput leaves FFT(gradOutput) in the plan (have_out; not for tiled plans, whose two
+        // passes window gradOutput differently)
+        return acc_grad_parameters(p, input, grad_output, grad_weight, grad_bias, scale, true, stream);
+    }
+    // Untiled: both passes share FFT(gradOutput) and have the same FFT size, so each stage is one grid:
+    // the (up to) three forward transforms, the two contractions, the two inverse transforms.  Every
+    // plane and every frequency goes through the code its own pass would run.
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const fbfc_conv_desc &d = p->d;
+    const pass_geom &gb = p->bprop, &ga = p->accgrad;
+    const int N = p->info.fft_size;
+    const int QH = fbfc::hermitian_count(N);
+    const fbfc::FreqMap fm = fbfc::hermitian_map(N);
+    StageTimer tm(p, s);
+    const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)gb.vbatch * d.out_planes, gb.a_h, gb.a_w,
+                               gb.a_pad_u, gb.a_pad_l, gb.a_win, 1};
+    const fbfc::FwdArgs fw = weight_args(p, weight);
+    const fbfc::FwdArgs fin = {input, p->in_freq, (long)ga.vbatch * d.in_planes, ga.a_h, ga.a_w, ga.a_pad_u,
+                               ga.a_pad_l, ga.a_win, 1};
+    const bool need_w = !((p->reuse & FBFC_REUSE_WEIGHT) && p->have_w);
+    const bool need_in = !((p->reuse & FBFC_REUSE_INPUT) && p->have_in);
+    if (need_w && need_in) {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_triple(N, fgo, fw, fin, s), "rfft2d(gradOutput, weight, input)");
+    } else if (need_w) {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_pair(N, fgo, fw, s), "rfft2d(gradOutput, weight)");
+    } else if (need_in) {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_pair(N, fgo, fin, s), "rfft2d(gradOutput, input)");
+    } else {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fgo, s), "rfft2d(gradOutput)");
+    }
+    tm.done(FBFC_STAGE_FFT_A);
+    p->have_in = p->have_w = true;
+    const float norm = 1.0f / ((float)N * (float)N);
+    // GI[b][p] = 1/N^2 sum_f GO[b][f] W[f][p];  GW[f][p] = scale/N^2 sum_b conj(GO[b][f]) I[b][p]
+    // (SpatialConvolutionFBFFT.lua:244-251, 337-344)
+    const fbfc::MmArgs mgi = {p->out_freq, p->w_freq, p->bw_gi, gb.vbatch, d.in_planes, d.out_planes, norm, 0};
+    const fbfc::MmArgs mgw = {p->out_freq, p->in_freq, p->bw_gw, d.out_planes, d.in_planes, ga.vbatch,
+                              scale * norm, 0};
+    FBFC_STAGE(tm, fbfc::launch_cgemm_backward(mgi, mgw, QH, fm, s), "cgemm(bprop, accGrad)");
+    tm.done(FBFC_STAGE_MM);
+    const fbfc::InvArgs igi = {p->bw_gi, grad_input, (long)gb.vbatch * d.in_planes, gb.r_h, gb.r_w, gb.r_pad_u,
+                               gb.r_pad_l, nullptr, 1, gb.r_win, nullptr, nullptr, 0.0f, 0, 0};
+    fbfc::InvArgs igw = {p->bw_gw, grad_weight, (long)d.out_planes * d.in_planes, ga.r_h, ga.r_w, 0, 0, nullptr, 1,
+                         {}, nullptr, nullptr, 0.0f, 0, 0};
+    if (grad_bias != nullptr) {
+        igw.go_freq = p->out_freq;
+        igw.grad_bias = grad_bias;
+        igw.scale = scale;
+        igw.batch = ga.vbatch;
+        igw.out_planes = d.out_planes;
+    }
+    FBFC_STAGE(tm, fbfc::launch_irfft2d_two(N, igi, igw, s), "irfft2d(gradInput, gradWeight) + bias grad");
+    tm.done(FBFC_STAGE_IFFT);
+    p->have_out = false;
+    return tm.finish();
 }
 
 static int fft2d_impl(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,

@@ -271,8 +271,29 @@ __device__ __forceinline__ void lds_direct_tile(const float2 *__restrict__ Mq, i
     }
 }
 
+// s_waitcnt vmcnt(n) alone (expcnt and lgkmcnt left at their maxima)
+template <int n>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(n >= 0 && n < 64, "vmcnt is a 6-bit field");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+}
+
+// Workgroup barrier without the memory fence of __syncthreads().  The fence makes the compiler put a
+// wait for every outstanding vector-memory operation in front of the barrier; the tile loop states its
+// own, narrower, condition: this wave's loads of the next tile have landed (wait_vmcnt) and its LDS reads
+// of the current tile have returned (lgkmcnt(0)).  The "memory" clobber keeps the compiler from moving LDS
+// accesses across.  Measured: 130 x 128x1024x1024 916 -> 883 us, 130 x 128x1024x512 502 -> 473 us.
+__device__ __forceinline__ void tile_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // One 64 x (32 WN) tile by 2 x WN waves, workgroup index wg = frequency * tiles + tile.
-// lds: A tiles (8 KB) and B tiles (4 WN KB), double-buffered.
+// lds: A tiles (8 KB) and B tiles (4 WN KB), double-buffered: the next tile lands while this one is
+// multiplied.  Measured alternatives that did not pay: a ring of three or four tiles in flight (the
+// loop never waits for a load: 0.03 us of 16.5 us at 144 x 128^3; 21.4 -> 21.7 / 24.1 us), and two
+// wave groups per tile that each take half of K to double the waves per SIMD (21.2 -> 24.9 us).
 template <int MODE, int WN>
 __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restrict__ A,
                                                const float2 *__restrict__ B, float2 *__restrict__ C,
@@ -318,8 +339,8 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
     };
 
     issue(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-    __syncthreads();
+    wait_vmcnt<0>();
+    tile_barrier();
 
     const int arow = 32 * wm + li, bcol = 32 * wn + li;
     // swizzled position of 16-byte chunk c of a K-contiguous row: 8-row block, row in block, c ^ row
@@ -365,8 +386,8 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
             }
         }
         if (kt + 1 < nk) {
-            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's share of the next tile is in LDS
-            __syncthreads();                     // ... and everyone's; nobody still reads the other buffer
+            wait_vmcnt<0>();  // this lane's share of the next tile is in LDS
+            tile_barrier();   // ... and everyone's; nobody still reads the other buffer
         }
     }
 
@@ -654,58 +675,41 @@ void cgemm_force_variant(int v) { g_force_variant.store(v); }
 static int splitk_override() { return g_force_variant.load(std::memory_order_relaxed); }
 
 
-template <int MODE>
-static hipError_t launch_mode(const float *A, const float *B, float *C, int n_freq, int m, int n,
-                              int k, float alpha, int accumulate, FreqMap fm, hipStream_t s)
+// Which kernel a problem takes (measured on MI355X):
+//  * a few rounds of 64x64 tiles whose last round would fill at most half the chip: whole rounds as
+//    LDS-direct tiles, the rest as split blocks (25 vs 31 us at 144 x 128^3, 28.4 vs 30.5 at
+//    544 x 128x64x64; with a fuller last round plain tiles are as fast);
+//  * N a multiple of 96 but not of 64 (96 input planes): 64x96 tiles by six waves.  At 2112 frequencies
+//    256x96x64 conj(A)^T B takes 293 us against 321 for the register-fed kernel, but 64x96x256 A B 290
+//    against 279, so the plain product keeps the register-fed kernel;
+//  * at least 4 full 64x64 tiles per CU and 64-aligned M, N: LDS-direct tiles;
+//  * otherwise, if M, N are multiples of 32 and K of 16: the register-fed kernel, with more
+//    waves sharing one block's K range the fewer blocks there are per SIMD;
+//  * anything else: register-staged LDS tiles with bounds checks.
+enum Variant { V_INVALID, V_HYBRID, V_TILES96, V_SPLIT4, V_SPLIT2, V_SPLIT1, V_TILES, V_STAGED };
+struct Choice {
+    Variant v;
+    int q_direct;  // V_HYBRID: frequencies [0, q_direct) as tiles, the rest as split blocks
+};
+
+static Choice choose_variant(int mode, const float *A, const float *B, int n_freq, int m, int n, int k)
 {
     const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
     const long total = (long)n_freq * tilesM * tilesN;
-    if (total <= 0 || total > 0x7fffff00L) return hipErrorInvalidValue;
-    // Kernel choice (measured on MI355X):
-    //  * at least 4 full 64x64 tiles per CU and 64-aligned M, N: LDS-direct tiles;
-    //  * otherwise, if M, N are multiples of 32 and K of 16: the register-fed kernel, with more
-    //    waves sharing one block's K range the fewer blocks there are per SIMD;
-    //  * anything else: register-staged LDS tiles with bounds checks.
+    if (total <= 0 || total > 0x7fffff00L) return {V_INVALID, 0};
     const bool aligned16 = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
     const int force = splitk_override();
     const bool direct_ok = (m % 64) == 0 && (n % 64) == 0 && (k % 16) == 0 && aligned16;
     const long tot32 = (long)n_freq * (m / 32) * (n / 32);
-    // A few rounds of tiles whose last round would fill at most half the chip: whole rounds as tiles,
-    // the rest as split blocks (measured: 25 vs 31 us at 144 x 128^3, 28.4 vs 30.5 at 544 x 128x64x64;
-    // with a fuller last round plain tiles are as fast).
     if (direct_ok && (k % 64) == 0 &&
         (force == 9 || (force < 0 && total >= 256 && total < 8 * 256 && total % 256 <= 128))) {
         const int t64 = tilesM * tilesN;
         const int q_direct = (int)((total / 256) * 256 / t64);
-        const int q_split = n_freq - q_direct;
-        if (q_split > 0 && q_direct > 0) {
-            const int direct_wgs = q_direct * t64;
-            const int split_tiles = q_split * (m / 32) * (n / 32);  // one workgroup per 32x32 block
-            const int chunk_direct = (direct_wgs + 7) / 8, chunk_split = (split_tiles + 7) / 8;
-            note_kernel("cgemm_hybrid_kernel", MODE, -1, (long)(chunk_direct + chunk_split) * 8 * 256);
-            hipLaunchKernelGGL(cgemm_hybrid_kernel<MODE>, dim3((unsigned)((chunk_direct + chunk_split) * 8)),
-                               dim3(256), 0, s, reinterpret_cast<const float2 *>(A),
-                               reinterpret_cast<const float2 *>(B), reinterpret_cast<float2 *>(C), m, n, k,
-                               alpha, accumulate, q_direct, direct_wgs, chunk_direct, split_tiles,
-                               split_tiles, chunk_split, fm);
-            return hipGetLastError();
-        }
+        if (n_freq - q_direct > 0 && q_direct > 0) return {V_HYBRID, q_direct};
     }
-    // N a multiple of 96 but not of 64 (config 5: 96 input planes): 64x96 tiles by six waves.  Measured
-    // at 2112 frequencies: 256x96x64 conj(A)^T B 293 us against 321 for the register-fed kernel, but
-    // 64x96x256 A B 290 against 279, so the plain product keeps the register-fed kernel.
-    if ((MODE != 1 || force == 8) && (m % 64) == 0 && (n % 96) == 0 && (n % 64) != 0 && (k % 16) == 0 && aligned16 &&
-        (force == 8 || (force < 0 && (long)n_freq * (m / 64) * (n / 96) >= 4 * 256))) {
-        const int t96 = n / 96;
-        const long tot = (long)n_freq * tilesM * t96;
-        const int ch = (int)((tot + 7) / 8);
-        note_kernel("cgemm_ldsdirect_kernel", MODE, 3, (long)ch * 8 * 384);
-        hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 3>), dim3((unsigned)(ch * 8)), dim3(384), 0, s,
-                           reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
-                           reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, t96, (int)tot, ch,
-                           fm);
-        return hipGetLastError();
-    }
+    if ((mode != 1 || force == 8) && (m % 64) == 0 && (n % 96) == 0 && (n % 64) != 0 && (k % 16) == 0 && aligned16 &&
+        (force == 8 || (force < 0 && (long)n_freq * (m / 64) * (n / 96) >= 4 * 256)))
+        return {V_TILES96, 0};
     const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && total >= 4 * 256));
     if (!prefer_direct && (m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 &&
         tot32 * 4 < 0x7fffff00L) {
@@ -714,25 +718,150 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
         else if (tot32 < 4 * 1024 && (k % 64) == 0) sk = 4;
         else if (tot32 < 8 * 1024 && (k % 32) == 0) sk = 2;
         else sk = 1;
-                if (sk == 4 && (k % 64) == 0) return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
-        if (sk == 2 && (k % 32) == 0) return launch_splitk<MODE, 2>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
-        if (sk == 1) return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        if (sk == 4 && (k % 64) == 0) return {V_SPLIT4, 0};
+        if (sk == 2 && (k % 32) == 0) return {V_SPLIT2, 0};
+        if (sk == 1) return {V_SPLIT1, 0};
     }
+    if (direct_ok && force != 0) return {V_TILES, 0};
+    return {V_STAGED, 0};
+}
+
+template <int MODE>
+static hipError_t launch_mode(const float *A, const float *B, float *C, int n_freq, int m, int n,
+                              int k, float alpha, int accumulate, FreqMap fm, hipStream_t s)
+{
+    const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
+    const long total = (long)n_freq * tilesM * tilesN;
+    const Choice ch = choose_variant(MODE, A, B, n_freq, m, n, k);
+    const float2 *A2 = reinterpret_cast<const float2 *>(A), *B2 = reinterpret_cast<const float2 *>(B);
+    float2 *C2 = reinterpret_cast<float2 *>(C);
     const int chunk = (int)((total + 7) / 8);
-    if (direct_ok && force != 0) {
-        note_kernel("cgemm_ldsdirect_kernel", MODE, 2, (long)chunk * 8 * 256);
-        hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 2>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
-                           reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
-                           reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
-                           (int)total, chunk, fm);
-        return hipGetLastError();
+    switch (ch.v) {
+        case V_HYBRID: {
+            const int t64 = tilesM * tilesN;
+            const int direct_wgs = ch.q_direct * t64;
+            const int split_tiles = (n_freq - ch.q_direct) * (m / 32) * (n / 32);  // one workgroup per 32x32 block
+            const int chunk_direct = (direct_wgs + 7) / 8, chunk_split = (split_tiles + 7) / 8;
+            note_kernel("cgemm_hybrid_kernel", MODE, -1, (long)(chunk_direct + chunk_split) * 8 * 256);
+            hipLaunchKernelGGL(cgemm_hybrid_kernel<MODE>, dim3((unsigned)((chunk_direct + chunk_split) * 8)),
+                               dim3(256), 0, s, A2, B2, C2, m, n, k, alpha, accumulate, ch.q_direct, direct_wgs,
+                               chunk_direct, split_tiles, split_tiles, chunk_split, fm);
+            return hipGetLastError();
+        }
+        case V_TILES96: {
+            const int t96 = n / 96;
+            const long tot = (long)n_freq * tilesM * t96;
+            const int c96 = (int)((tot + 7) / 8);
+            note_kernel("cgemm_ldsdirect_kernel", MODE, 3, (long)c96 * 8 * 384);
+            hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 3>), dim3((unsigned)(c96 * 8)), dim3(384), 0, s, A2, B2,
+                               C2, m, n, k, alpha, accumulate, tilesM, t96, (int)tot, c96, fm);
+            return hipGetLastError();
+        }
+        case V_SPLIT4: return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        case V_SPLIT2: return launch_splitk<MODE, 2>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        case V_SPLIT1: return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
+        case V_TILES:
+            note_kernel("cgemm_ldsdirect_kernel", MODE, 2, (long)chunk * 8 * 256);
+            hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 2>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s, A2,
+                               B2, C2, m, n, k, alpha, accumulate, tilesM, tilesN, (int)total, chunk, fm);
+            return hipGetLastError();
+        case V_STAGED:
+            note_kernel("cgemm_freq_kernel", MODE, -1, (long)chunk * 8 * 256);
+            hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s, A2, B2, C2, m,
+                               n, k, alpha, accumulate, tilesM, tilesN, (int)total, chunk, fm);
+            return hipGetLastError();
+        default: return hipErrorInvalidValue;
     }
-    note_kernel("cgemm_freq_kernel", MODE, -1, (long)chunk * 8 * 256);
-    hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
-                       reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
-                       reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tilesM, tilesN,
-                       (int)total, chunk, fm);
-    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------
+// The two contractions of a backward pass (A B for gradInput, conj(A)^T B for gradWeight) as one
+// grid: the tiles of both problems first, then the split blocks of both.  Each problem is cut into
+// tiles and blocks exactly as its own launch would cut it and runs the same code, so the results are
+// those of two launches; what is saved is one launch and one partly filled last round.
+// ---------------------------------------------------------------------------------------
+struct MmJob {
+    const float2 *A, *B;
+    float2 *C;
+    int M, N, K;
+    float alpha;
+    int accumulate;
+    int q_direct, direct_wgs, chunk_direct;  // frequencies [0, q_direct) as 64x64 tiles
+    int split_tiles, chunk_split;            // the rest as 32x32 blocks, K split over four waves
+};
+
+__global__ __launch_bounds__(256) void cgemm_backward_kernel(MmJob j1, MmJob j2, FreqMap fm)
+{
+    __shared__ __align__(16) float lds[LDSDIRECT_FLOATS];
+    const int x = (int)(blockIdx.x % 8);
+    int j = (int)(blockIdx.x / 8);
+    if (j < j1.chunk_direct) {
+        const int wg = x * j1.chunk_direct + j;
+        if (wg >= j1.direct_wgs) return;
+        ldsdirect_body<1, 2>(lds, j1.A, j1.B, j1.C, j1.M, j1.N, j1.K, j1.alpha, j1.accumulate, j1.M / 64,
+                             j1.N / 64, wg, 0, fm);
+        return;
+    }
+    j -= j1.chunk_direct;
+    if (j < j2.chunk_direct) {
+        const int wg = x * j2.chunk_direct + j;
+        if (wg >= j2.direct_wgs) return;
+        ldsdirect_body<2, 2>(lds, j2.A, j2.B, j2.C, j2.M, j2.N, j2.K, j2.alpha, j2.accumulate, j2.M / 64,
+                             j2.N / 64, wg, 0, fm);
+        return;
+    }
+    j -= j2.chunk_direct;
+    if (j < j1.chunk_split) {
+        const int wg = x * j1.chunk_split + j;
+        if (wg >= j1.split_tiles) return;
+        splitk_body<1, 4>(reinterpret_cast<float (*)[32][64]>(lds), j1.A, j1.B, j1.C, j1.M, j1.N, j1.K, j1.alpha,
+                          j1.accumulate, j1.M / 32, j1.N / 32, j1.split_tiles, wg, j1.q_direct, fm);
+        return;
+    }
+    j -= j1.chunk_split;
+    const int wg = x * j2.chunk_split + j;
+    if (wg >= j2.split_tiles) return;
+    splitk_body<2, 4>(reinterpret_cast<float (*)[32][64]>(lds), j2.A, j2.B, j2.C, j2.M, j2.N, j2.K, j2.alpha,
+                      j2.accumulate, j2.M / 32, j2.N / 32, j2.split_tiles, wg, j2.q_direct, fm);
+}
+
+// false: this problem's kernel is not one the grouped grid runs
+static bool make_mm_job(int mode, const MmArgs &a, int n_freq, MmJob &j)
+{
+    const Choice ch = choose_variant(mode, a.A, a.B, n_freq, a.m, a.n, a.k);
+    int q_direct;
+    if (ch.v == V_HYBRID) q_direct = ch.q_direct;
+    else if (ch.v == V_TILES) q_direct = n_freq;
+    else if (ch.v == V_SPLIT4) q_direct = 0;
+    else return false;
+    j.A = reinterpret_cast<const float2 *>(a.A);
+    j.B = reinterpret_cast<const float2 *>(a.B);
+    j.C = reinterpret_cast<float2 *>(a.C);
+    j.M = a.m; j.N = a.n; j.K = a.k;
+    j.alpha = a.alpha;
+    j.accumulate = a.accumulate;
+    j.q_direct = q_direct;
+    j.direct_wgs = q_direct * (a.m / 64) * (a.n / 64);
+    j.chunk_direct = (j.direct_wgs + 7) / 8;
+    j.split_tiles = (n_freq - q_direct) * (a.m / 32) * (a.n / 32);
+    j.chunk_split = (j.split_tiles + 7) / 8;
+    return true;
+}
+
+hipError_t launch_cgemm_backward(const MmArgs &gi, const MmArgs &gw, int n_freq, FreqMap fm, hipStream_t s)
+{
+    MmJob j1, j2;
+    if (make_mm_job(1, gi, n_freq, j1) && make_mm_job(2, gw, n_freq, j2)) {
+        const long chunks = (long)j1.chunk_direct + j2.chunk_direct + j1.chunk_split + j2.chunk_split;
+        if (chunks * 8 < 0x7fffff00L) {
+            kernel_log_add("cgemm_backward_kernel", chunks * 8 * 256);
+            hipLaunchKernelGGL(cgemm_backward_kernel, dim3((unsigned)(chunks * 8)), dim3(256), 0, s, j1, j2, fm);
+            return hipGetLastError();
+        }
+    }
+    const hipError_t e = launch_mode<1>(gi.A, gi.B, gi.C, n_freq, gi.m, gi.n, gi.k, gi.alpha, gi.accumulate, fm, s);
+    if (e != hipSuccess) return e;
+    return launch_mode<2>(gw.A, gw.B, gw.C, n_freq, gw.m, gw.n, gw.k, gw.alpha, gw.accumulate, fm, s);
 }
 
 hipError_t launch_cgemm_freq_map(int mode, const float *A, const float *B, float *C, int n_freq, FreqMap fm,

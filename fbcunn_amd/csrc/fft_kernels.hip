@@ -178,30 +178,36 @@ __device__ __forceinline__ void copy_windows(float *smem, float *g, const int4 *
 // the inputs that are known to be zero.
 template <int N, bool WIN, int NZ, bool RAW>
 __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<N, false, (NZ < N)>::MIN_WAVES)) void rfft2d_kernel(FwdJob job0, FwdJob job1,
-                                                                      unsigned blocks0)
+                                                                      FwdJob job2, unsigned blocks0,
+                                                                      unsigned blocks01)
 {
     using S = FftShape<N, false, (NZ < N)>;
     constexpr int T = S::T;
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x;
     const unsigned v = blockIdx.x;
-    const bool second = v >= blocks0;
-    const float *__restrict__ in = second ? job1.in : job0.in;
-    float2 *__restrict__ out = second ? job1.out : job0.out;
-    const long planes = second ? job1.planes : job0.planes;
-    const int h = second ? job1.h : job0.h, w = second ? job1.w : job0.w;
-    const int padU = second ? job1.padU : job0.padU, padL = second ? job1.padL : job0.padL;
-    const int vec4 = second ? job1.vec4 : job0.vec4;
-    const int herm = second ? job1.herm : job0.herm;
-    [[maybe_unused]] const Window &win = second ? job1.win : job0.win;
-    long x0 = plane_group<T>(v - (second ? blocks0 : 0u)) * T;
+    // up to three tensors per launch: workgroups [0, blocks0) work on job 0, [blocks0, blocks01) on
+    // job 1, the rest on job 2
+    const bool second = v >= blocks0, third = v >= blocks01;
+    const FwdJob &job = third ? job2 : (second ? job1 : job0);
+    const unsigned vfirst = third ? blocks01 : (second ? blocks0 : 0u);
+    const float *__restrict__ in = job.in;
+    float2 *__restrict__ out = job.out;
+    const long planes = job.planes;
+    const int h = job.h, w = job.w;
+    const int padU = job.padU, padL = job.padL;
+    const int vec4 = job.vec4;
+    const int herm = job.herm;
+    [[maybe_unused]] const Window &win = job.win;
+    const int job_tbl_off = job.tbl_off;
+    long x0 = plane_group<T>(v - vfirst) * T;
     if constexpr (WIN) {
-        if (win.remap) x0 = window_block<T>(v - (second ? blocks0 : 0u), win) * T;
+        if (win.remap) x0 = window_block<T>(v - vfirst, win) * T;
     }
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
-    [[maybe_unused]] int4 *tbl = reinterpret_cast<int4 *>(smem + (second ? job1.tbl_off : job0.tbl_off));
+    [[maybe_unused]] int4 *tbl = reinterpret_cast<int4 *>(smem + job_tbl_off);
     if constexpr (WIN) {
         if (win.on) build_window_table<N>(tbl, win, x0, planes, tid);
     }
@@ -409,12 +415,9 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
 // real[r][s] = y[r+padU][s+padL] (+ bias[plane % bias_period])
 // ---------------------------------------------------------------------------------
 template <int N, bool WIN, int PHASES = 0>
-__global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftShape<N, true, false, PHASES>::MIN_WAVES)) void irfft2d_kernel(const float2 *__restrict__ in,
-                                                      float *__restrict__ out, long planes,
-                                                      int h, int w, int padU, int padL,
-                                                      const float *__restrict__ bias,
-                                                      int bias_period, int vec4, BiasGradJob bgrad,
-                                                      unsigned bgrad_blocks, Window win, int tbl_off)
+__global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftShape<N, true, false, PHASES>::MIN_WAVES)) void irfft2d_kernel(InvJob job0, InvJob job1,
+                                                      unsigned blocks0, BiasGradJob bgrad,
+                                                      unsigned bgrad_blocks)
 {
     using S = FftShape<N, true, false, PHASES>;
     constexpr int T = S::T;
@@ -426,9 +429,19 @@ __global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftSh
         return;
     }
     const int tid = threadIdx.x;
-    long x0 = plane_group<T>(blockIdx.x - bgrad_blocks) * T;
+    const unsigned v = blockIdx.x - bgrad_blocks;
+    const bool second = v >= blocks0;
+    const InvJob &job = second ? job1 : job0;
+    const float2 *__restrict__ in = job.in;
+    float *__restrict__ out = job.out;
+    const long planes = job.planes;
+    const int h = job.h, w = job.w, padU = job.padU, padL = job.padL;
+    const float *__restrict__ bias = job.bias;
+    const int bias_period = job.bias_period, vec4 = job.vec4, tbl_off = job.tbl_off;
+    [[maybe_unused]] const Window &win = job.win;
+    long x0 = plane_group<T>(v - (second ? blocks0 : 0u)) * T;
     if constexpr (WIN) {
-        if (win.remap) x0 = window_block<T>(blockIdx.x - bgrad_blocks, win) * T;
+        if (win.remap) x0 = window_block<T>(v - (second ? blocks0 : 0u), win) * T;
     }
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
@@ -614,26 +627,34 @@ static bool window_ok(const Window &w, long planes, int h, int ww)
            w.img_h > 0 && w.img_w > 0 && h > 0 && ww > 0 && planes % ((long)w.nt * w.d1) == 0;
 }
 
-// second == nullptr: one tensor only
+// second == nullptr: one tensor only; third only with second
 // raw staging needs odd plane sizes (see the kernel) in every operand of the launch
 static bool raw_ok(const FwdArgs &a) { return (a.h & 1) && (a.w & 1) && !a.win.on; }
 
 template <int N, bool WIN, int NZ, bool RAW>
-static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
+static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipStream_t s,
+                                  const FwdArgs *third = nullptr)
 {
     size_t lds = fft_lds_bytes<N, false, (NZ < N)>(a.h, a.w, a.padU);
     const long blocks0 = fwd_blocks<N>(a.planes);
-    long blocks = blocks0;
+    long blocks01 = blocks0, blocks = blocks0;
     FwdJob j0 = make_job<N, (NZ < N)>(a);
-    FwdJob j1 = j0;
+    FwdJob j1 = j0, j2 = j0;
     if (second != nullptr) {
         const size_t lds1 = fft_lds_bytes<N, false, (NZ < N)>(second->h, second->w, second->padU);
         if (lds1 > lds) lds = lds1;
-        blocks += fwd_blocks<N>(second->planes);
+        blocks01 += fwd_blocks<N>(second->planes);
+        blocks = blocks01;
         j1 = make_job<N, (NZ < N)>(*second);
+        if (third != nullptr) {
+            const size_t lds2 = fft_lds_bytes<N, false, (NZ < N)>(third->h, third->w, third->padU);
+            if (lds2 > lds) lds = lds2;
+            blocks += fwd_blocks<N>(third->planes);
+            j2 = make_job<N, (NZ < N)>(*third);
+        }
     }
     if (WIN) {  // the window table sits behind the tile / staging area
-        j0.tbl_off = j1.tbl_off = (int)(lds / sizeof(float));
+        j0.tbl_off = j1.tbl_off = j2.tbl_off = (int)(lds / sizeof(float));
         lds += FftShape<N>::T * sizeof(int4);
     }
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
@@ -643,34 +664,70 @@ static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipSt
         kernel_log_add(name, blocks * FftShape<N, false, (NZ < N)>::THREADS);
     }
     hipLaunchKernelGGL((rfft2d_kernel<N, WIN, NZ, RAW>), dim3((unsigned)blocks), dim3(FftShape<N, false, (NZ < N)>::THREADS), lds, s, j0, j1,
-                       (unsigned)blocks0);
+                       j2, (unsigned)blocks0, (unsigned)blocks01);
     return hipGetLastError();
 }
 
 template <int N, bool WIN, int NZ = N>
-static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
+static hipError_t launch_fwd(const FwdArgs &a, const FwdArgs *second, hipStream_t s, const FwdArgs *third = nullptr)
 {
     if constexpr (!WIN && N <= 64) {
-        if (raw_ok(a) && (second == nullptr || raw_ok(*second))) return launch_fwd_impl<N, WIN, NZ, true>(a, second, s);
+        if (raw_ok(a) && (second == nullptr || raw_ok(*second)) && (third == nullptr || raw_ok(*third)))
+            return launch_fwd_impl<N, WIN, NZ, true>(a, second, s, third);
     }
-    return launch_fwd_impl<N, WIN, NZ, false>(a, second, s);
+    return launch_fwd_impl<N, WIN, NZ, false>(a, second, s, third);
 }
 
 template <int N, bool WIN, int PHASES>
-static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s)
+static InvJob make_inv_job(const InvArgs &a)
+{
+    using S = FftShape<N, true, false, PHASES>;
+    InvJob j;
+    j.in = reinterpret_cast<const float2 *>(a.in);
+    j.out = a.out;
+    j.planes = a.planes;
+    j.h = a.h; j.w = a.w; j.padU = a.padU; j.padL = a.padL;
+    j.bias = a.bias;
+    j.bias_period = a.bias_period > 0 ? a.bias_period : 1;
+    // every copy-out round starts TP planes after the previous one: all of them 16-byte aligned
+    j.vec4 = ((reinterpret_cast<uintptr_t>(a.out) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
+    j.tbl_off = 0;
+    j.win = a.win;
+    j.win.remap = window_remap_ok<S::T>(a.win, a.planes);
+    return j;
+}
+
+// second == nullptr: one tensor only.  The bias-gradient job, if any, is taken from `a` or `second`.
+template <int N, bool WIN, int PHASES>
+static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s, const InvArgs *second = nullptr)
 {
     using S = FftShape<N, true, false, PHASES>;
     size_t lds = fft_lds_bytes<N, true, false, PHASES>(a.h, a.w, a.padU);
-    const int tbl_off = (int)(lds / sizeof(float));
-    if (WIN) lds += S::T * sizeof(int4);
-    long blocks = (a.planes + S::T - 1) / S::T;
-    if (S::T * 8 < 128) blocks = (blocks + 15) / 16 * 16;  // whole cycles of the paired mapping
-    // every copy-out round starts TP planes after the previous one: all of them 16-byte aligned
-    const int vec4 = ((reinterpret_cast<uintptr_t>(a.out) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
-    Window win = a.win;
-    win.remap = window_remap_ok<S::T>(a.win, a.planes);
-    const BiasGradJob bgrad = {reinterpret_cast<const float2 *>(a.go_freq), a.grad_bias, a.scale, a.batch,
-                               a.out_planes};
+    auto nblocks = [](long planes) {
+        long b = (planes + S::T - 1) / S::T;
+        if (S::T * 8 < 128) b = (b + 15) / 16 * 16;  // whole cycles of the paired mapping
+        return b;
+    };
+    const long blocks0 = nblocks(a.planes);
+    long blocks = blocks0;
+    InvJob j0 = make_inv_job<N, WIN, PHASES>(a);
+    InvJob j1 = j0;
+    const InvArgs *bg = (a.go_freq != nullptr) ? &a : nullptr;
+    if (second != nullptr) {
+        const size_t lds1 = fft_lds_bytes<N, true, false, PHASES>(second->h, second->w, second->padU);
+        if (lds1 > lds) lds = lds1;
+        blocks += nblocks(second->planes);
+        j1 = make_inv_job<N, WIN, PHASES>(*second);
+        if (bg == nullptr && second->go_freq != nullptr) bg = second;
+    }
+    if (WIN) {
+        j0.tbl_off = j1.tbl_off = (int)(lds / sizeof(float));
+        lds += S::T * sizeof(int4);
+    }
+    BiasGradJob bgrad = {nullptr, nullptr, 0.0f, 0, 0};
+    if (bg != nullptr)
+        bgrad = BiasGradJob{reinterpret_cast<const float2 *>(bg->go_freq), bg->grad_bias, bg->scale, bg->batch,
+                            bg->out_planes};
     const unsigned bblocks = (bgrad.dc != nullptr) ? bias_grad_dc_blocks(bgrad.planes) : 0u;
     if (blocks + bblocks > 0x7fffffffL) return hipErrorInvalidValue;
     {
@@ -679,8 +736,7 @@ static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s)
         kernel_log_add(name, (blocks + bblocks) * S::THREADS);
     }
     hipLaunchKernelGGL((irfft2d_kernel<N, WIN, PHASES>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
-                       reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL,
-                       a.bias, a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks, win, tbl_off);
+                       j0, j1, (unsigned)blocks0, bgrad, bblocks);
     return hipGetLastError();
 }
 
@@ -810,6 +866,24 @@ hipError_t launch_rfft2d_pair(int N, const FwdArgs &a, const FwdArgs &b, hipStre
     return dispatch_fwd(N, a, &b, s);
 }
 
+// Three forward transforms of one size: one launch where one kernel takes all three operands
+// (N <= 32, no windows), otherwise a pair and a single one.
+hipError_t launch_rfft2d_triple(int N, const FwdArgs &a, const FwdArgs &b, const FwdArgs &c, hipStream_t s)
+{
+    // every operand keeps the staging variant it gets in a pair or alone: all three agree on it
+    const bool plain = !a.win.on && !b.win.on && !c.win.on && raw_ok(a) == raw_ok(b) && raw_ok(b) == raw_ok(c);
+    if (plain && planes_ok(N, a.planes) && planes_ok(N, b.planes) && planes_ok(N, c.planes)) {
+        switch (N) {
+            case 8: return launch_fwd<8, false>(a, &b, s, &c);
+            case 16: return launch_fwd<16, false>(a, &b, s, &c);
+            case 32: return launch_fwd<32, false>(a, &b, s, &c);
+            default: break;
+        }
+    }
+    const hipError_t e = dispatch_fwd(N, a, &b, s);
+    return e != hipSuccess ? e : dispatch_fwd(N, c, nullptr, s);
+}
+
 hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s)
 {
     if (!planes_ok(N, a.planes) || !window_ok(a.win, a.planes, a.h, a.w)) return hipErrorInvalidValue;
@@ -829,6 +903,27 @@ hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s)
         case 128: return launch_irfft2d_large(N, a, s);
         default: return hipErrorInvalidValue;
     }
+}
+
+// Two inverse transforms of one size: one launch for N <= 32 without windows, two otherwise.
+hipError_t launch_irfft2d_two(int N, const InvArgs &a, const InvArgs &b, hipStream_t s)
+{
+    if (!a.win.on && !b.win.on && planes_ok(N, a.planes) && planes_ok(N, b.planes)) {
+        switch (N) {
+            case 8: return launch_inv_impl<8, false, 0>(a, s, &b);
+            case 16: return launch_inv_impl<16, false, 0>(a, s, &b);
+            case 32: {
+                // each tensor keeps the kernel it would get alone; one launch if that is the same kernel
+                const long two_rounds = 2L * 512 * FftShape<32, true>::T;
+                const bool pa = a.planes > two_rounds, pb = b.planes > two_rounds;
+                if (pa != pb) break;
+                return pa ? launch_inv_impl<32, false, 2>(a, s, &b) : launch_inv_impl<32, false, 0>(a, s, &b);
+            }
+            default: break;
+        }
+    }
+    const hipError_t e = launch_irfft2d_args(N, a, s);
+    return e != hipSuccess ? e : launch_irfft2d_args(N, b, s);
 }
 
 hipError_t launch_irfft2d(int N, const float *in, float *out, long planes, int h, int w, int padU,

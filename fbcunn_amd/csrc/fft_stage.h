@@ -188,4 +188,17 @@ struct FwdJob {
     Window win;
 };
 
+// One launch of the inverse kernel can produce two tensors of the same FFT size (the two inverse
+// transforms of backward()): workgroups [0, blocks0) work on job 0, the rest on job 1.
+struct InvJob {
+    const float2 *in;
+    float *out;
+    long planes;
+    int h, w, padU, padL;
+    const float *bias;
+    int bias_period, vec4;
+    int tbl_off;
+    Window win;
+};
+
 }  // namespace fbfc

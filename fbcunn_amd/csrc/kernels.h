@@ -56,6 +56,10 @@ struct InvArgs {
     int batch, out_planes;
 };
 hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s);
+// backward(): its three forward transforms and its two inverse transforms as one launch each where one
+// kernel takes them all (N <= 32, no windows), as several launches otherwise; same results either way
+hipError_t launch_rfft2d_triple(int N, const FwdArgs &a, const FwdArgs &b, const FwdArgs &c, hipStream_t s);
+hipError_t launch_irfft2d_two(int N, const InvArgs &a, const InvArgs &b, hipStream_t s);
 
 // Largest number of planes one launch of an N x N transform takes (the kernels address a frequency
 // row of the spectrum with 32-bit byte offsets): floor((2^31 - 1) / ((N/2 + 1) * 8)).
@@ -101,6 +105,17 @@ inline FreqMap hermitian_map(int N) { return FreqMap{(N / 2 + 1) * (N / 2 + 1), 
 inline int hermitian_count(int N) { return (N / 2 + 1) * (N / 2 + 1) + (N / 2 - 1) * (N / 2 - 1); }
 hipError_t launch_cgemm_freq_map(int mode, const float *A, const float *B, float *C, int n_freq, FreqMap fm,
                                  int m, int n, int k, float alpha, int accumulate, hipStream_t s);
+// The two contractions of a backward pass, C1 = A1 B1 (mode 1) and C2 = conj(A2)^T B2 (mode 2), over the
+// same frequencies: one launch where both problems take tile / split-block kernels, two otherwise; the
+// results are those of two launch_cgemm_freq_map calls either way.
+struct MmArgs {
+    const float *A, *B;
+    float *C;
+    int m, n, k;
+    float alpha;
+    int accumulate;
+};
+hipError_t launch_cgemm_backward(const MmArgs &gi, const MmArgs &gw, int n_freq, FreqMap fm, hipStream_t s);
 
 // Launch log of the calling thread: every kernel launcher appends "<kernel name> grid=<work-items>";
 // the pass entry points clear it before a stage and keep what the stage logged.

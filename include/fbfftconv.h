@@ -134,7 +134,12 @@ int fbfc_acc_grad_parameters(fbfc_plan *plan, const float *input, const float *g
  * updateGradInput followed by accGradParameters, the second reusing the spectrum of
  * gradOutput the first one computed (the reference passes its outputTransposeBuffer in the
  * reuse list) whatever the plan's reuse policy.  Tiled plans recompute it (their two passes
- * window gradOutput differently).  Results equal those of the two separate calls. */
+ * window gradOutput differently).  Results equal those of the two separate calls, bit for bit.
+ * For an untiled plan each stage of the two passes is issued as one grid (the forward
+ * transforms of gradOutput, weight and input; both contractions; both inverse transforms with
+ * the bias gradient), which needs the two product spectra in buffers of their own: the first
+ * call allocates input_freq_bytes + weight_freq_bytes more device memory and keeps it until
+ * the plan is destroyed.  If that allocation fails the pass runs as its two halves. */
 int fbfc_backward(fbfc_plan *plan, const float *input, const float *grad_output, const float *weight,
                   float *grad_input, float *grad_weight, float *grad_bias, float scale, void *stream);
 

@@ -289,6 +289,54 @@ def test_backward_equals_the_two_passes(nn, oracle, cls, extra):
     b.cleanupBuffers()
 
 
+# (B, P, F, k, H, pad, reuse, what the contraction stage must have launched)
+_GROUPED = [
+    (128, 128, 128, 3, 13, 1, None, "cgemm_backward_kernel"),    # N = 16: tiles + split blocks of both problems
+    (128, 128, 128, 3, 13, 1, "all", "cgemm_backward_kernel"),
+    (64, 64, 64, 5, 27, 2, None, "cgemm_backward_kernel"),       # N = 32
+    (64, 64, 128, 3, 13, 0, None, "cgemm_backward_kernel"),      # split blocks only + tiles and blocks
+    (16, 96, 64, 3, 14, 1, None, "cgemm_"),                      # 96 planes, even sizes: whatever kernels fit
+    (8, 32, 32, 9, 57, 0, None, "cgemm_"),                       # N = 64: stages of several launches
+]
+
+
+@pytest.mark.parametrize("B,P,F,k,H,pad,reuse,mm", _GROUPED)
+def test_backward_one_grid_per_stage(nn, B, P, F, k, H, pad, reuse, mm):
+    """An untiled backward() issues each stage of its two passes as one grid where one kernel can
+    take them all (SpatialConvolutionFFT.lua:405-416 only orders the passes): bit-equal to the two
+    passes run one after the other, with and without buffer reuse, and again on a second call."""
+    x = synth.uniform(91, (B, P, H, H), stream=0)
+    w = synth.normal(91, (F, P, k, k), 0.0, 0.05, stream=1)
+    oh = H + 2 * pad - k + 1
+    xd = dev(x)
+    kw = {} if reuse is None else {"memoryReusePolicy": reuse}
+    a = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad, **kw)
+    b = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad, **kw)
+    for net in (a, b):
+        net.weight.copy_(dev(w))
+    for it in range(2):
+        g = synth.uniform(92 + it, (B, F, oh, oh), stream=3)
+        gd = dev(g)
+        for net in (a, b):
+            net.gradWeight.fill_(float("nan"))
+            net.gradBias.fill_(float("nan"))
+            net.updateOutput(xd)     # with reuse: leaves the spectra of input and weight in the plan
+        gin = host(a.backward(xd, gd, 0.7))
+        stages = a.stageKernels(xd)
+        b.updateGradInput(xd, gd)
+        b.accGradParameters(xd, gd, 0.7)
+        assert np.isfinite(gin).all()
+        assert np.array_equal(gin, host(b.gradInput)), "gradInput, call %d" % it
+        assert np.array_equal(host(a.gradWeight), host(b.gradWeight)), "gradWeight, call %d" % it
+        assert np.array_equal(host(a.gradBias), host(b.gradBias)), "gradBias, call %d" % it
+        assert mm in stages["mm"], stages
+        if mm == "cgemm_backward_kernel":
+            # one launch per stage
+            assert all(v.count("grid=") == 1 for v in stages.values()), stages
+    a.cleanupBuffers()
+    b.cleanupBuffers()
+
+
 def test_backward_between_other_passes(nn, oracle):
     """backward() reuses the spectrum updateGradInput leaves in the plan: with other passes and
     changing inputs around it, every result must still be the one of the current inputs."""
