@@ -367,6 +367,22 @@ def measure_copy_bandwidth(torch):
     return {"ms": ms, "GBps_read_plus_write": 2 * a.numel() * 4 / (ms * 1e-3) / 1e9}
 
 
+def measure_mfma_clock(nn, torch):
+    """The shader clock the tile contraction kernel runs at (clock counters inside the kernel), for the main
+    workload's contraction shape and for a wide one that keeps the matrix pipes busy for milliseconds.
+    The published fp32 MFMA peak assumes the 2.4 GHz peak clock."""
+    out = {"peak_clock_mhz": 2400.0}
+    for name, (Q, m, n, k, launches) in {"config4_contraction": (130, 128, 128, 128, 20),
+                                         "wide_contraction_130x128x1024x1024": (130, 128, 1024, 1024, 5)}.items():
+        A = torch.rand(Q, m, k, 2, device="cuda") - 0.5
+        B = torch.rand(Q, n, k, 2, device="cuda") - 0.5
+        C = torch.empty(Q, m, n, 2, device="cuda")
+        mhz = nn.contractionClock(0, A, B, C, launches=launches)
+        out[name] = {"mhz": mhz, "fp32_mfma_peak_at_this_clock_tflops": MFMA_FP32_PEAK_TF * mhz / 2400.0}
+        del A, B, C
+    return out
+
+
 def cpu_baseline(synth):
     """The CPU oracle on the main workload: the whole batch-128 training step
     (three passes, 19.1 GFLOP of direct convolution), all host threads OpenMP
@@ -476,6 +492,12 @@ def main():
     line["reuse_all_step"] = measure_reuse_step(nn, torch, synth, args.steps, args.warmup)
     line["fprop_plus_backward_step"] = measure_backward_step(nn, torch, synth, args.steps, args.warmup)
     line["copy_256MiB"] = measure_copy_bandwidth(torch)
+    line["mfma_clock"] = measure_mfma_clock(nn, torch)
+    if "mfma_issued_frac" in roofline:
+        # the same utilisation against the matrix peak at the clock the kernel was measured to run at
+        c = line["mfma_clock"]["config4_contraction"]["mhz"]
+        roofline["mfma_clock_mhz"] = c
+        roofline["mfma_issued_frac_at_measured_clock"] = roofline["mfma_issued_frac"] * 2400.0 / c if c > 0 else None
     # the other stated configurations, compact
     configs = {}
     for name in CONFIGS:

@@ -471,6 +471,31 @@ int fbfc_debug_force_contraction_kernel(int variant)
     return FBFC_OK;
 }
 
+int fbfc_debug_contraction_clock(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
+                                 int k, int launches, float *mhz, void *stream)
+{
+    if (A == nullptr || B == nullptr || C == nullptr || mhz == nullptr || launches < 1)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned long long *ticks = nullptr;
+    FBFC_TRY(hipMalloc(reinterpret_cast<void **>(&ticks), 2 * sizeof *ticks), "hipMalloc");
+    hipError_t e = hipSuccess;
+    // the clock settles over the run of launches: the last one is the one read
+    for (int i = 0; i < launches && e == hipSuccess; ++i) {
+        if (i == launches - 1) e = hipMemsetAsync(ticks, 0, 2 * sizeof *ticks, s);
+        if (e == hipSuccess) e = fbfc::launch_cgemm_clock_probe(mode, A, B, C, n_freq, m, n, k, ticks, s);
+    }
+    unsigned long long h[2] = {0, 0};
+    if (e == hipSuccess) e = hipMemcpyAsync(h, ticks, sizeof h, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(ticks);
+    if (e == hipErrorInvalidValue)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "the clock probe takes m, n multiples of 64 and k of 16");
+    if (e != hipSuccess) return fail_hip(e, "contraction clock probe");
+    *mhz = h[1] ? (float)((double)h[0] / ((double)h[1] / 100.0)) : 0.0f;
+    return FBFC_OK;
+}
+
 int fbfc_plan_stage_ms(const fbfc_plan *p, float *ms, int n)
 {
     if (p == nullptr || ms == nullptr || n < 0) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");

@@ -439,6 +439,29 @@ __global__ __launch_bounds__(128 * WN) void cgemm_ldsdirect_kernel(const float2 
     ldsdirect_body<MODE, WN>(lds, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, wg, 0, fm);
 }
 
+// Measurement variant of the 64x64 tile kernel: each workgroup also adds the shader-clock ticks
+// (s_memtime) and the 100 MHz ticks (s_memrealtime) it lived for to ticks[0] and ticks[1]; their ratio
+// is the clock the kernel actually ran at.  Under sustained fp32 MFMA load the chip settles well below its
+// 2.4 GHz peak clock, which is what the MFMA roofline is quoted at.
+template <int MODE>
+__global__ __launch_bounds__(256) void cgemm_ldsdirect_clock_kernel(const float2 *__restrict__ A,
+                                                                    const float2 *__restrict__ B,
+                                                                    float2 *__restrict__ C, int M, int N,
+                                                                    int K, float alpha, int tilesM, int tilesN,
+                                                                    int total_wgs, int chunk,
+                                                                    unsigned long long *ticks)
+{
+    __shared__ __align__(16) float lds[ldsdirect_floats(2)];
+    const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
+    if (wg >= total_wgs) return;
+    const long long c0 = clock64(), w0 = wall_clock64();
+    ldsdirect_body<MODE, 2>(lds, A, B, C, M, N, K, alpha, 0, tilesM, tilesN, wg, 0, FreqMap{0, 1, 0});
+    if (threadIdx.x == 0) {
+        atomicAdd(ticks, (unsigned long long)(clock64() - c0));
+        atomicAdd(ticks + 1, (unsigned long long)(wall_clock64() - w0));
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // Split-K kernel for small problems (few 64x64 tiles per CU).
 //
@@ -875,6 +898,27 @@ hipError_t launch_cgemm_backward(const MmArgs &gi, const MmArgs &gw, int n_freq,
     const hipError_t e = launch_mode<1>(gi.A, gi.B, gi.C, n_freq, gi.m, gi.n, gi.k, gi.alpha, gi.accumulate, fm, s);
     if (e != hipSuccess) return e;
     return launch_mode<2>(gw.A, gw.B, gw.C, n_freq, gw.m, gw.n, gw.k, gw.alpha, gw.accumulate, fm, s);
+}
+
+hipError_t launch_cgemm_clock_probe(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
+                                    int k, unsigned long long *ticks, hipStream_t s)
+{
+    if (mode < 0 || mode > 2 || (m % 64) != 0 || (n % 64) != 0 || (k % 16) != 0 || m <= 0 || n <= 0 || k <= 0)
+        return hipErrorInvalidValue;
+    if (((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) != 0) return hipErrorInvalidValue;
+    const int tilesM = m / 64, tilesN = n / 64;
+    const long total = (long)n_freq * tilesM * tilesN;
+    if (total <= 0 || total > 0x7fffff00L) return hipErrorInvalidValue;
+    const int chunk = (int)((total + 7) / 8);
+    const float2 *A2 = reinterpret_cast<const float2 *>(A), *B2 = reinterpret_cast<const float2 *>(B);
+    float2 *C2 = reinterpret_cast<float2 *>(C);
+    const dim3 grid((unsigned)(chunk * 8)), block(256);
+    switch (mode) {
+        case 0: hipLaunchKernelGGL(cgemm_ldsdirect_clock_kernel<0>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
+        case 1: hipLaunchKernelGGL(cgemm_ldsdirect_clock_kernel<1>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
+        default: hipLaunchKernelGGL(cgemm_ldsdirect_clock_kernel<2>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
+    }
+    return hipGetLastError();
 }
 
 hipError_t launch_cgemm_freq_map(int mode, const float *A, const float *B, float *C, int n_freq, FreqMap fm,

@@ -126,6 +126,10 @@ const char *kernel_log_get();
 // 9 = hybrid of LDS-direct tiles and split blocks, 1 / 2 / 4 = register-fed kernel with that many
 // waves per block (falls back to the shape rule where the forced variant cannot run the shape).
 void cgemm_force_variant(int v);
+// The 64x64 tile kernel with clock counters: adds every workgroup's shader-clock and 100 MHz ticks to
+// ticks[0] and ticks[1] (m, n multiples of 64, k of 16)
+hipError_t launch_cgemm_clock_probe(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
+                                    int k, unsigned long long *ticks, hipStream_t s);
 
 // layout_kernels.hip: frequency-major freq[q][plane] <-> the reference's plane-major buf[plane][q].
 // mode 0: same frequency order; 1: buf[a][c] = X[ky = c][kx = a] (fbfft for N < 8 or N > 32);

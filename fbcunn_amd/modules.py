@@ -541,6 +541,25 @@ def transposeMM(A, B, C, invNorm, conjugateTransposeA, conjugateTransposeB, accu
     return C
 
 
+def contractionClock(mode, A, B, C, launches=20):
+    """Shader clock (MHz) the 64x64 tile contraction kernel runs at over `launches` back-to-back launches
+    of C = op(A, B) (mode 0: A conj(B)^T, 1: A B, 2: conj(A)^T B; operands (Q, rows, cols, 2) as for
+    transposeMM); C receives the unscaled product.  A measurement aid: the MFMA peak is quoted at the
+    chip's peak clock, sustained fp32 MFMA work runs below it."""
+    for t, nme in ((A, "A"), (B, "B"), (C, "C")):
+        _check_tensor(t, nme, 4)
+    Q, m, n = C.size(0), C.size(1), C.size(2)
+    k = A.size(1) if mode == 2 else A.size(2)
+    exp_a = (Q, k, m, 2) if mode == 2 else (Q, m, k, 2)
+    exp_b = (Q, n, k, 2) if mode == 0 else (Q, k, n, 2)
+    if mode not in (0, 1, 2) or tuple(A.shape) != exp_a or tuple(B.shape) != exp_b:
+        raise ValueError("operand shapes do not match: A %s B %s C %s" % (tuple(A.shape), tuple(B.shape), tuple(C.shape)))
+    mhz = ctypes.c_float(0.0)
+    check(lib().fbfc_debug_contraction_clock(mode, _ptr(A), _ptr(B), _ptr(C), Q, m, n, k, int(launches),
+                                             ctypes.byref(mhz), _stream()))
+    return float(mhz.value)
+
+
 def updateOutputBias(output, bias):
     """updateOutputBiasFFI (src/ConvolutionBias.cu:256-260); like the reference's kernel it takes
     non-contiguous tensors (test/BiasTest.cpp:38-63)."""

@@ -178,6 +178,16 @@ int fbfc_plan_stage_kernel(const fbfc_plan *plan, int stage, char *name, size_t 
  * 8 = LDS-direct tiles, 9 = LDS-direct tiles plus split blocks, 1 / 2 / 4 = register-fed kernel
  * with that many waves per block.  A variant that cannot run a shape falls back to the shape rule. */
 int fbfc_debug_force_contraction_kernel(int variant);
+/* Measurement (no counterpart in the reference): the shader clock the 64x64 tile contraction kernel
+ * actually runs at.  Issues `launches` back-to-back launches of the per-frequency product with clock
+ * counters in the kernel and returns, for the last launch, shader-clock ticks per microsecond of
+ * workgroup lifetime in *mhz.  mode 0: C = A conj(B)^T with A (Q, m, k), B (Q, n, k) (updateOutput);
+ * mode 1: C = A B with B (Q, k, n) (updateGradInput); mode 2: C = conj(A)^T B with A (Q, k, m),
+ * B (Q, k, n) (accGradParameters); C (Q, m, n) is written unscaled.  m, n multiples of 64, k of 16,
+ * 16-byte aligned operands.  The MFMA peak is quoted at the 2.4 GHz peak clock; under sustained fp32 MFMA load the chip
+ * runs lower, and this is the number that says how much lower.  Synchronises the stream. */
+int fbfc_debug_contraction_clock(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
+                                 int k, int launches, float *mhz, void *stream);
 
 /* Stand-alone stages ------------------------------------------------------------
  * Replaces FFTWrapper_fft with fbfft (src/fft/FFTWrapperLua.cpp:209-272 ->

@@ -124,3 +124,23 @@ def test_transpose_mm_on_the_reference_operand_layout(nn, mode):
         got = got[..., 0] + 1j * got[..., 1]
         exp = 0.5 * want + (C0 if accumulate else 0)
         assert np.abs(got - exp).max() <= 2e-5 * np.abs(exp).max()
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_contraction_clock_probe(nn, mode):
+    """The measurement variant of the tile kernel: same product as transposeMM (it runs the same tile code),
+    and a shader clock between the chip's idle and peak clocks."""
+    Q, m, n, k = 40, 128, 64, 64
+    A = synth.uniform(5, (Q, k, m, 2) if mode == 2 else (Q, m, k, 2))
+    B = synth.uniform(6, (Q, n, k, 2) if mode == 0 else (Q, k, n, 2))
+    C = torch.full((Q, m, n, 2), float("nan"), device="cuda")
+    want = torch.empty_like(C)
+    nn.transposeMM(dev(A), dev(B), want, 1.0, mode == 2, mode == 0, False)
+    mhz = nn.contractionClock(mode, dev(A), dev(B), C, launches=5)
+    assert 300.0 < mhz < 2600.0, mhz
+    got, ref = _c(host(C)), _c(host(want))
+    assert np.isfinite(got).all()
+    assert np.abs(got - ref).max() <= TOL * np.abs(ref).max()
+    with pytest.raises(nn.FbfcError):
+        nn.contractionClock(mode, dev(A)[:, :, :40].contiguous() if mode != 2 else dev(A)[:, :40].contiguous(),
+                            dev(B)[:, :, :40].contiguous() if mode == 0 else dev(B)[:, :40].contiguous(), C)
