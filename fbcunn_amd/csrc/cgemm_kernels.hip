@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
 //     different bank groups (XOR swizzle instead of row padding);
 //   row-contiguous tile [16 k][32 chunks]: one instruction = 2 rows, stored as they lie.
 // ---------------------------------------------------------------------------------------
-// ROWS = rows of a K-contiguous tile resp. columns of a row-contiguous one (64 or 96): ROWS / 8 blocks
+// ROWS = rows of a K-contiguous tile resp. columns of a row-contiguous one (64 or 32): ROWS / 8 blocks
 // of 1 KB, dealt round-robin to the NW waves of the workgroup.
 template <bool KC, int ROWS, int NW>
 __device__ __forceinline__ void lds_direct_tile(const float2 *__restrict__ Mq, int ld, int r0, int c0,
@@ -424,7 +424,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
 constexpr int ldsdirect_floats(int wn) { return 2 * (64 * KT * 2 + 32 * wn * KT * 2); }
 constexpr int LDSDIRECT_FLOATS = ldsdirect_floats(2);  // 32 KB
 
-// WN = 2: 64x64 tiles, 256 lanes.  WN = 3: 64x96 tiles, 384 lanes (N a multiple of 96 but not of 64).
+// WN = 2: 64x64 tiles, 256 lanes.  WN = 1: 64x32 tiles, 128 lanes (N a multiple of 96 but not of 64).
 template <int MODE, int WN>
 __global__ __launch_bounds__(128 * WN) void cgemm_ldsdirect_kernel(const float2 *__restrict__ A,
                                                                   const float2 *__restrict__ B,
@@ -715,14 +715,14 @@ static int splitk_override() { return g_force_variant.load(std::memory_order_rel
 //  * a few rounds of 64x64 tiles whose last round would fill at most half the chip: whole rounds as
 //    LDS-direct tiles, the rest as split blocks (25 vs 31 us at 144 x 128^3, 28.4 vs 30.5 at
 //    544 x 128x64x64; with a fuller last round plain tiles are as fast);
-//  * N a multiple of 96 but not of 64 (96 input planes): 64x96 tiles by six waves.  At 2112 frequencies
-//    256x96x64 conj(A)^T B takes 293 us against 321 for the register-fed kernel, but 64x96x256 A B 290
-//    against 279, so the plain product keeps the register-fed kernel;
+//  * N a multiple of 96 but not of 64 (96 input planes): 64x32 tiles by two waves.  At 2112 frequencies
+//    256x96x64 conj(A)^T B takes 268 us (284 with 64x96 tiles by six waves, 321 with the register-fed
+//    kernel); 64x96x256 A B is as fast either way (251 us) and keeps the register-fed kernel;
 //  * at least 4 full 64x64 tiles per CU and 64-aligned M, N: LDS-direct tiles;
 //  * otherwise, if M, N are multiples of 32 and K of 16: the register-fed kernel, with more
 //    waves sharing one block's K range the fewer blocks there are per SIMD;
 //  * anything else: register-staged LDS tiles with bounds checks.
-enum Variant { V_INVALID, V_HYBRID, V_TILES96, V_SPLIT4, V_SPLIT2, V_SPLIT1, V_TILES, V_STAGED };
+enum Variant { V_INVALID, V_HYBRID, V_TILES32, V_SPLIT4, V_SPLIT2, V_SPLIT1, V_TILES, V_STAGED };
 struct Choice {
     Variant v;
     int q_direct;  // V_HYBRID: frequencies [0, q_direct) as tiles, the rest as split blocks
@@ -745,7 +745,7 @@ static Choice choose_variant(int mode, const float *A, const float *B, int n_fre
     }
     if ((mode != 1 || force == 8) && (m % 64) == 0 && (n % 96) == 0 && (n % 64) != 0 && (k % 16) == 0 && aligned16 &&
         (force == 8 || (force < 0 && (long)n_freq * (m / 64) * (n / 96) >= 4 * 256)))
-        return {V_TILES96, 0};
+        return {V_TILES32, 0};
     const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && total >= 4 * 256));
     if (!prefer_direct && (m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 &&
         tot32 * 4 < 0x7fffff00L) {
@@ -784,13 +784,13 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
                                chunk_direct, split_tiles, split_tiles, chunk_split, fm);
             return hipGetLastError();
         }
-        case V_TILES96: {
-            const int t96 = n / 96;
-            const long tot = (long)n_freq * tilesM * t96;
-            const int c96 = (int)((tot + 7) / 8);
-            note_kernel("cgemm_ldsdirect_kernel", MODE, 3, (long)c96 * 8 * 384);
-            hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 3>), dim3((unsigned)(c96 * 8)), dim3(384), 0, s, A2, B2,
-                               C2, m, n, k, alpha, accumulate, tilesM, t96, (int)tot, c96, fm);
+        case V_TILES32: {
+            const int t32 = n / 32;
+            const long tot = (long)n_freq * tilesM * t32;
+            const int c32 = (int)((tot + 7) / 8);
+            note_kernel("cgemm_ldsdirect_kernel", MODE, 1, (long)c32 * 8 * 128);
+            hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 1>), dim3((unsigned)(c32 * 8)), dim3(128), 0, s, A2, B2,
+                               C2, m, n, k, alpha, accumulate, tilesM, t32, (int)tot, c32, fm);
             return hipGetLastError();
         }
         case V_SPLIT4: return launch_splitk<MODE, 4>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);

@@ -32,7 +32,7 @@ SHAPES = [  # Q, m, n, k
     # a few rounds of 64x64 tiles with a ragged last one: whole rounds as LDS-direct tiles, the
     # left-over frequencies as split blocks, in one launch
     (70, 128, 128, 64), (300, 64, 64, 128), (33, 192, 128, 64),
-    # N a multiple of 96 but not of 64 and at least 1024 tiles: 64x96 tiles by six waves
+    # N a multiple of 96 but not of 64 and at least 1024 64x96 blocks: 64x32 tiles by two waves
     (1024, 64, 96, 16), (260, 128, 288, 32), (1100, 64, 96, 48),
 ]
 
