@@ -47,3 +47,40 @@ def test_passes_replay_from_a_graph(B, P, F, k, H, pad):
         for got, ref, name in zip(results(), want, ("output", "gradInput", "gradWeight", "gradBias")):
             assert np.array_equal(host(got), ref), "replay %d: %s differs from the eager result" % (rep, name)
     net.cleanupBuffers()
+
+
+@pytest.mark.parametrize("B,P,F,k,H,pad", [(64, 64, 128, 3, 13, 1), (4, 16, 48, 5, 27, 2)])
+def test_backward_replays_from_a_graph(B, P, F, k, H, pad):
+    """backward() with one grid per stage: its first call makes the two extra spectrum buffers, every
+    later call allocates nothing and can be captured."""
+    from fbcunn_amd import nn
+    o = H + 2 * pad - k + 1
+    net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad)
+    net.weight.copy_(dev(synth.normal(6, (F, P, k, k), 0.0, 0.05, stream=1)))
+    x, g = dev(synth.uniform(6, (B, P, H, H), stream=0)), dev(synth.uniform(6, (B, F, o, o), stream=3))
+
+    def step():
+        net.updateOutput(x)
+        net.backward(x, g, 0.5)
+
+    results = lambda: [net.output, net.gradInput, net.gradWeight, net.gradBias]
+    step()
+    torch.cuda.synchronize()
+    want = [host(t).copy() for t in results()]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        for t in results():
+            t.fill_(float("nan"))
+        (x * 2).sum().item()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref, name in zip(results(), want, ("output", "gradInput", "gradWeight", "gradBias")):
+            assert np.array_equal(host(got), ref), "replay %d: %s differs from the eager result" % (rep, name)
+    net.cleanupBuffers()
