@@ -899,7 +899,9 @@ hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s)
         case 8: return launch_inv<8, false>(a, s);
         case 16: return launch_inv<16, false>(a, s);
         case 32: return launch_inv<32, false>(a, s);
-        case 64: return a.planes <= kSmallLaunch64 ? launch_irfft2d_large(N, a, s) : launch_inv<64, false>(a, s);
+        case 64:
+            return (a.planes <= kSmallLaunch64 || (a.h <= 16 && a.w <= 16)) ? launch_irfft2d_large(N, a, s)
+                                                                             : launch_inv<64, false>(a, s);
         case 128: return launch_irfft2d_large(N, a, s);
         default: return hipErrorInvalidValue;
     }
