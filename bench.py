@@ -351,6 +351,31 @@ def measure_reference_list(nn, torch, synth, steps):
     return out
 
 
+def measure_spectrum_store_policy(nn, torch, synth, steps, warmup):
+    """The forward transforms leave a spectrum of up to 144 MB in the caches for the contraction (ordinary
+    stores) and stream a larger one past them (non-temporal stores).  Measured alone, 10 launches back to back,
+    the transform is faster with streaming stores; the pass is faster without.  Both ways, same layer, same run:
+    the main workload's step and its fprop FFT stage under the library's rule and with streaming forced on."""
+    from fbcunn_amd import _lib
+    cfg = CONFIGS[MAIN]
+    passes = cfg[6]
+    out = {}
+    for name, mode in (("by_size_rule", -1), ("always_streaming", 1)):
+        _lib.check(_lib.lib().fbfc_debug_force_spectrum_streaming(mode))
+        try:
+            net, x, g = make_layer(nn, torch, synth, cfg)
+            ms_step = time_loop(torch, lambda: [run_pass(net, x, g, p) for p in passes], max(steps, 100), max(warmup, 10))
+            warm, _ = stage_times(net, x, g, "fprop", STAGE_REPS, 3)
+            model = stage_model(cfg, "fprop", net._plan_for(cfg[0], cfg[3], cfg[3]).info.fft_size,
+                                net._plan_for(cfg[0], cfg[3], cfg[3]).info.n_freq)
+            out[name] = {"ms_per_step": ms_step, "fprop_fft_stage_ms": warm["fft"],
+                         "fprop_fft_stage_frac": model["fft"][1] / (warm["fft"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            net.cleanupBuffers()
+        finally:
+            _lib.check(_lib.lib().fbfc_debug_force_spectrum_streaming(-1))
+    return out
+
+
 def measure_copy_bandwidth(torch):
     """A plain 256 MiB device-to-device copy: what HBM delivers to a trivial kernel on this box."""
     a = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
@@ -493,6 +518,7 @@ def main():
     line["fprop_plus_backward_step"] = measure_backward_step(nn, torch, synth, args.steps, args.warmup)
     line["copy_256MiB"] = measure_copy_bandwidth(torch)
     line["mfma_clock"] = measure_mfma_clock(nn, torch)
+    line["spectrum_store_policy"] = measure_spectrum_store_policy(nn, torch, synth, args.steps, args.warmup)
     if "mfma_issued_frac" in roofline:
         # the same utilisation against the matrix peak at the clock the kernel was measured to run at
         c = line["mfma_clock"]["config4_contraction"]["mhz"]

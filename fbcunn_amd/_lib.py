@@ -61,6 +61,7 @@ SIGNATURES = {
     "fbfc_plan_stage_ms": (_i, [_vp, ctypes.POINTER(_f), _i]),
     "fbfc_plan_stage_kernel": (_i, [_vp, _i, ctypes.c_char_p, ctypes.c_size_t]),
     "fbfc_debug_force_contraction_kernel": (_i, [_i]),
+    "fbfc_debug_force_spectrum_streaming": (_i, [_i]),
     "fbfc_debug_contraction_clock": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, ctypes.POINTER(_f), _vp]),
     "fbfc_fft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp]),
     "fbfc_ifft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),

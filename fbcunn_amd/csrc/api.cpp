@@ -471,6 +471,13 @@ int fbfc_debug_force_contraction_kernel(int variant)
     return FBFC_OK;
 }
 
+int fbfc_debug_force_spectrum_streaming(int mode)
+{
+    if (mode < -1 || mode > 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "spectrum streaming mode must be -1, 0 or 1");
+    fbfc::spectrum_stream_force(mode);
+    return FBFC_OK;
+}
+
 int fbfc_debug_contraction_clock(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
                                  int k, int launches, float *mhz, void *stream)
 {

@@ -22,6 +22,7 @@
 // The inverse kernel is the mirror image and adds the bias while cropping.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdio>
 #include <mutex>
 
@@ -67,11 +68,13 @@ struct FftShape {
     static constexpr int LPR = THREADS / PH;
 };
 
+static std::atomic<int> g_stream_override{-1};
+int spectrum_stream_override() { return g_stream_override.load(std::memory_order_relaxed); }
+void spectrum_stream_force(int v) { g_stream_override.store(v); }
+
+// whether this kernel's runs per frequency are whole 128-byte lines
 template <int N>
-__device__ __forceinline__ void store_freq(float2 *p, const float2 &v)
-{
-    store_freq_run<(FftShape<N, false>::T * 8 >= 128)>(p, v);
-}
+constexpr bool whole_lines() { return FftShape<N, false>::T * 8 >= 128; }
 
 // Windowed operands: virtual plane v = (b * nt + tile) * d1 + c, so the workgroups of one tile (d1 / T of
 // them) are followed by those of the next tile -- on other XCDs, although neighbouring windows of one
@@ -385,28 +388,33 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
         const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + tc) * (long)sizeof(float2));
         char *obase = reinterpret_cast<char *>(out + x0);
         const long rowbytes = (long)S::NH * planes * (long)sizeof(float2);
-        if (kx != 0) {
-            static_for<N>([&](auto kk) {
-                constexpr int ky = decltype(kk)::value;
-                store_freq<N>(reinterpret_cast<float2 *>(obase + ky * rowbytes + voff),
-                         make_float2(re[brev<N>(ky)], im[brev<N>(ky)]));
-            });
-        } else {
-            // C = FFT(col0 + i colNyq), both real sequences: untangle
-            static_for<N>([&](auto kk) {
-                constexpr int ky = decltype(kk)::value;
-                constexpr int kn = (N - ky) % N;
-                const float zr = re[brev<N>(ky)], zi = im[brev<N>(ky)];
-                const float nr = re[brev<N>(kn)], ni = im[brev<N>(kn)];
-                // both columns are spectra of real sequences: rows above N/2 repeat rows below it
-                if (ky <= N / 2 || !herm) {
-                    store_freq<N>(reinterpret_cast<float2 *>(obase + ky * rowbytes + voff),
-                             make_float2(0.5f * (zr + nr), 0.5f * (zi - ni)));
-                    store_freq<N>(reinterpret_cast<float2 *>(obase + ky * rowbytes + vnyq),
-                             make_float2(0.5f * (zi + ni), 0.5f * (nr - zr)));
-                }
-            });
-        }
+        auto store_all = [&](auto stream_tag) {
+            constexpr bool STREAM = decltype(stream_tag)::value;
+            if (kx != 0) {
+                static_for<N>([&](auto kk) {
+                    constexpr int ky = decltype(kk)::value;
+                    store_freq_run<STREAM>(reinterpret_cast<float2 *>(obase + ky * rowbytes + voff),
+                                           make_float2(re[brev<N>(ky)], im[brev<N>(ky)]));
+                });
+            } else {
+                // C = FFT(col0 + i colNyq), both real sequences: untangle
+                static_for<N>([&](auto kk) {
+                    constexpr int ky = decltype(kk)::value;
+                    constexpr int kn = (N - ky) % N;
+                    const float zr = re[brev<N>(ky)], zi = im[brev<N>(ky)];
+                    const float nr = re[brev<N>(kn)], ni = im[brev<N>(kn)];
+                    // both columns are spectra of real sequences: rows above N/2 repeat rows below it
+                    if (ky <= N / 2 || !herm) {
+                        store_freq_run<STREAM>(reinterpret_cast<float2 *>(obase + ky * rowbytes + voff),
+                                               make_float2(0.5f * (zr + nr), 0.5f * (zi - ni)));
+                        store_freq_run<STREAM>(reinterpret_cast<float2 *>(obase + ky * rowbytes + vnyq),
+                                               make_float2(0.5f * (zi + ni), 0.5f * (nr - zr)));
+                    }
+                });
+            }
+        };
+        if (whole_lines<N>() && job.stream) store_all(std::true_type{});
+        else store_all(std::false_type{});
     }
 }
 
@@ -615,6 +623,7 @@ static FwdJob make_job(const FwdArgs &a)
     j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
     j.tbl_off = 0;
     j.herm = a.herm;
+    j.stream = stream_spectrum(a.planes, N);
     j.win = a.win;
     j.win.remap = window_remap_ok<S::T>(a.win, a.planes);
     return j;

@@ -119,6 +119,7 @@ rfft2d_rows_kernel(FwdJob job0, FwdJob job1, unsigned blocks0)
     const int padU = second ? job1.padU : job0.padU, padL = second ? job1.padL : job0.padL;
     const int vec4 = second ? job1.vec4 : job0.vec4;
     const int herm = second ? job1.herm : job0.herm;
+    const int stream = second ? job1.stream : job0.stream;
     const long x0 = plane_group<T, S::G>(v - (second ? blocks0 : 0u)) * T;
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
@@ -282,12 +283,16 @@ rfft2d_rows_kernel(FwdJob job0, FwdJob job1, unsigned blocks0)
         const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + tc) * (long)sizeof(float2));
         char *obase = reinterpret_cast<char *>(out + x0);
         const long rowbytes = (long)S::NH * planes * (long)sizeof(float2);
+        // non-temporal stores only for runs of whole lines, and only when the spectrum outgrows the caches
+        const bool nt = WHOLE && stream;
         if (role == 0) {
             fft_block_nz<M, 0, 0, 2, false, NZC>(re, im);
-            store_column<N, WHOLE, 0>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
+            if (nt) store_column<N, WHOLE, 0>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
+            else store_column<N, false, 0>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
         } else {
             fft_block_nz<M, 0, 1, 2, false, NZC>(re, im);
-            store_column<N, WHOLE, 1>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
+            if (nt) store_column<N, WHOLE, 1>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
+            else store_column<N, false, 1>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
         }
     }
 }
@@ -492,6 +497,7 @@ static FwdJob make_rows_job(const FwdArgs &a)
     j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
     j.tbl_off = 0;
     j.herm = a.herm;
+    j.stream = stream_spectrum(a.planes, N);
     j.win = a.win;
     return j;
 }

@@ -125,14 +125,28 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
     }
 }
 
-// Spectrum stores.  Runs of whole 128-byte lines (N <= 32) are streamed past the cache (measured: 8.3 ->
-// 6.9 us for the 16384-plane N = 16 transform); the half-line runs of N >= 64 rely on the L2 to join the
-// two workgroups that share a line and stay ordinary stores.
-template <bool WHOLE_LINES>
+// Spectrum stores.  STREAM: written past the caches with the non-temporal hint.  That pays for a
+// spectrum no cache will hold until the contraction reads it, and only for runs of whole 128-byte lines
+// (part-line runs rely on the L2 to join the workgroups that share a line); a smaller spectrum is better
+// left in the L2 and the 256 MB memory-side cache, where the contraction finds it.  Measured per training
+// step, non-temporal always / never / above the limit below: batch 128, 128 -> 128 planes, 13 x 13 (19 MB
+// per spectrum) 120.8 / 116.8 / 116.8 us; 64 -> 64, 27 x 27 forward pass (36 MB) 52.7 / 48.9 / 48.9 us;
+// 96 -> 256, 24 x 24 (53 / 107 / 142 MB) 615 / 588 / 587 us; 256 -> 512, 12 x 12 (38 / 151 / 75 MB)
+// 550 / 551 / 547 us; batch 64, 96 -> 256, 55 x 55 (104 / 415 / 277 MB) 1.381 / 1.407 / 1.375 ms.
+template <bool STREAM>
 __device__ __forceinline__ void store_freq_run(float2 *p, const float2 &v)
 {
-    if constexpr (WHOLE_LINES) store_nt(p, v);
+    if constexpr (STREAM) store_nt(p, v);
     else *p = v;
+}
+
+// the launchers' rule: planes * frequencies * 8 bytes of one operand's spectrum against what the caches keep
+constexpr long kStreamSpectrumBytes = 144L << 20;
+int spectrum_stream_override();  // -1: the rule; 0 / 1: never / always (a measurement knob)
+inline int stream_spectrum(long planes, int n)
+{
+    const int o = spectrum_stream_override();
+    return o >= 0 ? o : planes * (long)n * (n / 2 + 1) * 8 > kStreamSpectrumBytes;
 }
 
 // Raw staging for the forward transform: the chunk of nfloats contiguous floats at g goes to LDS as it
@@ -185,6 +199,7 @@ struct FwdJob {
     int h, w, padU, padL, vec4;
     int tbl_off;  // windowed operand: float offset of the window table in LDS
     int herm;     // leave out the entries (ky > N/2, kx in {0, N/2}): conjugates of (N - ky, kx)
+    int stream;   // non-temporal spectrum stores (kernels whose runs are whole lines)
     Window win;
 };
 

@@ -126,6 +126,8 @@ const char *kernel_log_get();
 // 9 = hybrid of LDS-direct tiles and split blocks, 1 / 2 / 4 = register-fed kernel with that many
 // waves per block (falls back to the shape rule where the forced variant cannot run the shape).
 void cgemm_force_variant(int v);
+// -1: spectra are stored non-temporally when they outgrow the caches (the rule); 0 / 1: never / always
+void spectrum_stream_force(int v);
 // The 64x64 tile kernel with clock counters: adds every workgroup's shader-clock and 100 MHz ticks to
 // ticks[0] and ticks[1] (m, n multiples of 64, k of 16)
 hipError_t launch_cgemm_clock_probe(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,

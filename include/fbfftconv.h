@@ -178,6 +178,12 @@ int fbfc_plan_stage_kernel(const fbfc_plan *plan, int stage, char *name, size_t 
  * 8 = LDS-direct tiles, 9 = LDS-direct tiles plus split blocks, 1 / 2 / 4 = register-fed kernel
  * with that many waves per block.  A variant that cannot run a shape falls back to the shape rule. */
 int fbfc_debug_force_contraction_kernel(int variant);
+/* Measurement knob (no counterpart in the reference): how the forward transforms store their spectra,
+ * for the whole process.  -1 = by size (default): a spectrum of more than 144 MB is written with
+ * non-temporal stores, a smaller one with ordinary stores so that the contraction finds it in the caches;
+ * 0 = never non-temporal; 1 = always (where the kernel writes whole 128-byte lines).  Results do not
+ * depend on it. */
+int fbfc_debug_force_spectrum_streaming(int mode);
 /* Measurement (no counterpart in the reference): the shader clock the 64x64 tile contraction kernel
  * actually runs at.  Issues `launches` back-to-back launches of the per-frequency product with clock
  * counters in the kernel and returns, for the last launch, shader-clock ticks per microsecond of

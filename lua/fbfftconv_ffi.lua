@@ -41,6 +41,7 @@ int fbfc_plan_set_timed(fbfc_plan *plan, int reps);
 int fbfc_plan_stage_ms(const fbfc_plan *plan, float *ms, int n);
 int fbfc_plan_stage_kernel(const fbfc_plan *plan, int stage, char *name, size_t n);
 int fbfc_debug_force_contraction_kernel(int variant);
+int fbfc_debug_force_spectrum_streaming(int mode);
 int fbfc_debug_contraction_clock(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
                                  int k, int launches, float *mhz, void *stream);
 int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
