@@ -623,7 +623,7 @@ static FwdJob make_job(const FwdArgs &a)
     j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
     j.tbl_off = 0;
     j.herm = a.herm;
-    j.stream = stream_spectrum(a.planes, N);
+    j.stream = stream_spectrum(a.planes, N, a.herm);
     j.win = a.win;
     j.win.remap = window_remap_ok<S::T>(a.win, a.planes);
     return j;
