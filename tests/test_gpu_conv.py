@@ -358,3 +358,30 @@ def test_backward_between_other_passes(nn, oracle):
         _close(host(net.gradBias), oracle.bias_acc_grad_parameters(g, 1.0), "gradBias %d" % it)
         _close(host(out2), oracle.cross_correlation_valid(x, w, (1, 1), p4), "output %d" % it)
     net.cleanupBuffers()
+
+
+def test_spectrum_store_policy_does_not_change_results(nn):
+    """How the forward transforms store their spectra (ordinary stores for the contraction to find in the caches,
+    or non-temporal ones) is a matter of speed only: all three passes are bit-identical either way."""
+    from fbcunn_amd import _lib
+    B, P, F, k, H, pad = 16, 32, 64, 3, 13, 1
+    x = dev(synth.uniform(71, (B, P, H, H), stream=0))
+    g = dev(synth.uniform(71, (B, F, H, H), stream=3))
+    w = dev(synth.normal(71, (F, P, k, k), 0.0, 0.05, stream=1))
+    results = []
+    try:
+        for mode in (0, 1, -1):
+            _lib.check(_lib.lib().fbfc_debug_force_spectrum_streaming(mode))
+            net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad)
+            net.weight.copy_(w)
+            net.bias.zero_()
+            out = host(net.updateOutput(x)).copy()
+            gin = host(net.updateGradInput(x, g)).copy()
+            net.accGradParameters(x, g, 1.0)
+            results.append((out, gin, host(net.gradWeight).copy(), host(net.gradBias).copy()))
+            net.cleanupBuffers()
+    finally:
+        _lib.check(_lib.lib().fbfc_debug_force_spectrum_streaming(-1))
+    for other in results[1:]:
+        for a, b in zip(results[0], other):
+            assert np.isfinite(a).all() and np.array_equal(a, b)
