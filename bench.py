@@ -357,15 +357,14 @@ def measure_reference_list(nn, torch, synth, steps):
 
 
 def measure_spectrum_store_policy(nn, torch, synth, steps, warmup):
-    """The forward transforms leave a spectrum of up to 144 MB in the caches for the contraction (ordinary
-    stores) and stream a larger one past them (non-temporal stores).  Measured alone, 10 launches back to back,
-    the transform is faster with streaming stores; the pass is faster without.  Both ways, same layer, same run:
-    the main workload's step and its fprop FFT stage under the library's rule and with streaming forced on."""
+    """The forward transforms write their spectra through to the memory side, whose cache keeps them for the
+    contraction; non-temporal stores stream them past it.  Measured alone the transform is as fast either way,
+    the step is not.  Both ways, same layer, same run: the main workload's step and its fprop FFT stage."""
     from fbcunn_amd import _lib
     cfg = CONFIGS[MAIN]
     passes = cfg[6]
     out = {}
-    for name, mode in (("by_size_rule", -1), ("always_streaming", 1)):
+    for name, mode in (("write_through", -1), ("non_temporal", 1)):
         _lib.check(_lib.lib().fbfc_debug_force_spectrum_streaming(mode))
         try:
             net, x, g = make_layer(nn, torch, synth, cfg)

@@ -473,7 +473,7 @@ int fbfc_debug_force_contraction_kernel(int variant)
 
 int fbfc_debug_force_spectrum_streaming(int mode)
 {
-    if (mode < -1 || mode > 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "spectrum streaming mode must be -1, 0 or 1");
+    if (mode != -1 && mode != 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "spectrum streaming mode must be -1 or 1");
     fbfc::spectrum_stream_force(mode);
     return FBFC_OK;
 }

@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
                 v.x += o.x;
                 v.y += o.y;
             }
-            store_nt(dst, v);
+            store_wt(dst, v);
         }
     }
 }
@@ -417,7 +417,7 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
             v.x += o.x;
             v.y += o.y;
         }
-        store_nt(dst, v);
+        store_wt(dst, v);
     }
 }
 
@@ -598,7 +598,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
                 v.x += o.x;
                 v.y += o.y;
             }
-            store_nt(dst, v);
+            store_wt(dst, v);
         }
     } else {
         // add the SK partial accumulators of a block: each of its waves finalises 16/SK registers
@@ -628,7 +628,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
                 v.x += o.x;
                 v.y += o.y;
             }
-            store_nt(dst, v);
+            store_wt(dst, v);
         }
     }
 }

@@ -388,8 +388,8 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
         const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + tc) * (long)sizeof(float2));
         char *obase = reinterpret_cast<char *>(out + x0);
         const long rowbytes = (long)S::NH * planes * (long)sizeof(float2);
-        auto store_all = [&](auto stream_tag) {
-            constexpr bool STREAM = decltype(stream_tag)::value;
+        auto store_all = [&](auto mode_tag) {
+            constexpr int STREAM = decltype(mode_tag)::value;
             if (kx != 0) {
                 static_for<N>([&](auto kk) {
                     constexpr int ky = decltype(kk)::value;
@@ -413,8 +413,7 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
                 });
             }
         };
-        if (whole_lines<N>() && job.stream) store_all(std::true_type{});
-        else store_all(std::false_type{});
+        with_store_mode<whole_lines<N>()>(job.stream, store_all);
     }
 }
 
@@ -623,7 +622,7 @@ static FwdJob make_job(const FwdArgs &a)
     j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
     j.tbl_off = 0;
     j.herm = a.herm;
-    j.stream = stream_spectrum(a.planes, N, a.herm);
+    j.stream = spectrum_store_mode();
     j.win = a.win;
     j.win.remap = window_remap_ok<S::T>(a.win, a.planes);
     return j;

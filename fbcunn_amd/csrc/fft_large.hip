@@ -58,7 +58,7 @@ struct RowShape {
 // forward: real (planes,h,w) -> freq [N*(N/2+1)][planes] complex
 // ---------------------------------------------------------------------------------
 // Stores the outputs ky = 2 k' + ROLE of one tile column (X[2 k' + ROLE] sits at brev(k')).
-template <int N, bool WHOLE, int ROLE>
+template <int N, int WHOLE, int ROLE>
 __device__ __forceinline__ void store_column(const float (&re)[N / 2], const float (&im)[N / 2], char *obase,
                                              long rowbytes, unsigned voff, unsigned vnyq, bool slot0, int herm)
 {
@@ -283,16 +283,16 @@ rfft2d_rows_kernel(FwdJob job0, FwdJob job1, unsigned blocks0)
         const unsigned vnyq = (unsigned)(((long)(N / 2) * planes + tc) * (long)sizeof(float2));
         char *obase = reinterpret_cast<char *>(out + x0);
         const long rowbytes = (long)S::NH * planes * (long)sizeof(float2);
-        // non-temporal stores only for runs of whole lines, and only when the spectrum outgrows the caches
-        const bool nt = WHOLE && stream;
         if (role == 0) {
             fft_block_nz<M, 0, 0, 2, false, NZC>(re, im);
-            if (nt) store_column<N, WHOLE, 0>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
-            else store_column<N, false, 0>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
+            with_store_mode<WHOLE>(stream, [&](auto mode_tag) {
+                store_column<N, decltype(mode_tag)::value, 0>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
+            });
         } else {
             fft_block_nz<M, 0, 1, 2, false, NZC>(re, im);
-            if (nt) store_column<N, WHOLE, 1>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
-            else store_column<N, false, 1>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
+            with_store_mode<WHOLE>(stream, [&](auto mode_tag) {
+                store_column<N, decltype(mode_tag)::value, 1>(re, im, obase, rowbytes, voff, vnyq, kx == 0, herm);
+            });
         }
     }
 }
@@ -497,7 +497,7 @@ static FwdJob make_rows_job(const FwdArgs &a)
     j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
     j.tbl_off = 0;
     j.herm = a.herm;
-    j.stream = stream_spectrum(a.planes, N, a.herm);
+    j.stream = spectrum_store_mode();
     j.win = a.win;
     return j;
 }

@@ -125,34 +125,33 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
     }
 }
 
-// Spectrum stores.  STREAM: written past the caches with the non-temporal hint.  That pays for a
-// spectrum no cache will hold until the contraction reads it, and only for runs of whole 128-byte lines
-// (part-line runs rely on the L2 to join the workgroups that share a line); a smaller spectrum is better
-// left in the L2 and the 256 MB memory-side cache, where the contraction finds it.  Measured per training
-// step, non-temporal always / never / above the limit below: batch 128, 128 -> 128 planes, 13 x 13 (19 MB
-// per spectrum) 120.8 / 116.8 / 116.8 us; 64 -> 64, 27 x 27 forward pass (36 MB) 52.7 / 48.9 / 48.9 us;
-// 96 -> 256, 24 x 24 (53 / 107 / 142 MB) 615 / 588 / 587 us; 256 -> 512, 12 x 12 (38 / 151 / 75 MB)
-// 550 / 551 / 547 us; batch 64, 96 -> 256, 55 x 55 (104 / 415 / 277 MB) 1.381 / 1.407 / 1.375 ms.
-template <bool STREAM>
+// Spectrum stores.  Kernels whose runs per frequency are whole 128-byte lines write them through
+// (store_nt.h), or non-temporally when the measurement knob says so; part-line runs rely on the L2 to join
+// the workgroups that share a line and stay ordinary stores (written through, 6144 planes of 55 x 55 at
+// N = 64 with 64-byte runs take 45.2 instead of 43.2 us, 4096 planes at N = 128 with 32-byte runs 216
+// instead of 187 us).
+enum SpectrumStore { STORE_WT = 0, STORE_NT = 1, STORE_ORDINARY = 2 };
+template <int MODE>
 __device__ __forceinline__ void store_freq_run(float2 *p, const float2 &v)
 {
-    if constexpr (STREAM) store_nt(p, v);
+    if constexpr (MODE == STORE_NT) store_nt(p, v);
+    else if constexpr (MODE == STORE_WT) store_wt(p, v);
     else *p = v;
 }
-
-// The launchers' rule.  in_pass: the transform belongs to a convolution pass, whose contraction reads the
-// spectrum next (those are the launches that leave out the redundant entries): planes * frequencies * 8 bytes
-// against what the caches keep.  A stand-alone transform has no known reader and is streamed: alone it
-// is 5-10 % faster that way (8192 planes of 32 x 32: 15.1 against 17.0 us), and a round trip through the
-// inverse takes the same time either way.
-constexpr long kStreamSpectrumBytes = 144L << 20;
-int spectrum_stream_override();  // -1: the rule; 0 / 1: never / always (a measurement knob)
-inline int stream_spectrum(long planes, int n, int in_pass)
+// calls body(integral_constant<int, mode>) with the run-time mode as a compile-time one
+template <bool WHOLE_LINES, class F>
+__device__ __forceinline__ void with_store_mode(int mode, F &&body)
 {
-    const int o = spectrum_stream_override();
-    if (o >= 0) return o;
-    return !in_pass || planes * (long)n * (n / 2 + 1) * 8 > kStreamSpectrumBytes;
+    if constexpr (!WHOLE_LINES) {
+        body(std::integral_constant<int, STORE_ORDINARY>{});
+    } else {
+        if (mode == STORE_NT) body(std::integral_constant<int, STORE_NT>{});
+        else body(std::integral_constant<int, STORE_WT>{});
+    }
 }
+
+int spectrum_stream_override();  // 1: non-temporal spectrum stores (a measurement knob); otherwise write-through
+inline int spectrum_store_mode() { return spectrum_stream_override() == 1 ? STORE_NT : STORE_WT; }
 
 // Raw staging for the forward transform: the chunk of nfloats contiguous floats at g goes to LDS as it
 // lies, by LDS-direct loads (global_load_lds): no staging registers, no LDS store instructions and no
@@ -204,7 +203,7 @@ struct FwdJob {
     int h, w, padU, padL, vec4;
     int tbl_off;  // windowed operand: float offset of the window table in LDS
     int herm;     // leave out the entries (ky > N/2, kx in {0, N/2}): conjugates of (N - ky, kx)
-    int stream;   // non-temporal spectrum stores (kernels whose runs are whole lines)
+    int stream;   // SpectrumStore: how the spectrum is written
     Window win;
 };
 

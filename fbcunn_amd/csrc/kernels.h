@@ -126,7 +126,7 @@ const char *kernel_log_get();
 // 9 = hybrid of LDS-direct tiles and split blocks, 1 / 2 / 4 = register-fed kernel with that many
 // waves per block (falls back to the shape rule where the forced variant cannot run the shape).
 void cgemm_force_variant(int v);
-// -1: spectra are stored non-temporally when they outgrow the caches (the rule); 0 / 1: never / always
+// -1: spectra are written through (default); 1: non-temporal stores where runs are whole lines
 void spectrum_stream_force(int v);
 // The 64x64 tile kernel with clock counters: adds every workgroup's shader-clock and 100 MHz ticks to
 // ticks[0] and ticks[1] (m, n multiples of 64, k of 16)

@@ -92,7 +92,7 @@ def test_plan_refuses_more_planes_than_one_launch_addresses():
 def test_debug_knob_validates_its_argument():
     assert _lib.lib().fbfc_debug_force_contraction_kernel(3) == _lib.ERR_INVALID_ARGUMENT
     assert _lib.lib().fbfc_debug_force_contraction_kernel(-1) == _lib.OK
-    assert _lib.lib().fbfc_debug_force_spectrum_streaming(2) == _lib.ERR_INVALID_ARGUMENT
+    assert _lib.lib().fbfc_debug_force_spectrum_streaming(0) == _lib.ERR_INVALID_ARGUMENT
     assert _lib.lib().fbfc_debug_force_spectrum_streaming(-1) == _lib.OK
 
 
