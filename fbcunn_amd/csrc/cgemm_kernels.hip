@@ -33,6 +33,16 @@ __device__ __forceinline__ int map_freq(int i, const FreqMap &fm)
     return fm.split + row * fm.nh + (j - row * fm.rowlen) + 1;
 }
 
+// The kernels' `accumulate` argument carries two flags.  A result the caches can keep until the inverse
+// transform reads it is written through to the memory side; a larger one is streamed with non-temporal
+// stores (same rule and numbers as the spectra of the forward transforms, fft_stage.h).
+constexpr int RESULT_ACCUMULATE = 1, RESULT_STREAM = 2;
+__device__ __forceinline__ void store_result(float2 *p, const float2 &v, int flags)
+{
+    if (flags & RESULT_STREAM) store_nt(p, v);
+    else store_wt(p, v);
+}
+
 constexpr int BM = 64, BN = 64, KT = 16;
 constexpr int LDK = 2 * KT + 4;  // floats per row of a K-contiguous tile [64][KT] (+16 B pad)
 constexpr int LDM = 2 * 64;      // floats per row of a row-contiguous tile [KT][64]
@@ -219,12 +229,12 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
         if (row < M && col < N) {
             float2 v = make_float2(alpha * cre[r], alpha * cim[r]);
             float2 *dst = Cq + (long)row * N + col;
-            if (accumulate) {
+            if (accumulate & RESULT_ACCUMULATE) {
                 const float2 o = *dst;
                 v.x += o.x;
                 v.y += o.y;
             }
-            store_wt(dst, v);
+            store_result(dst, v, accumulate);
         }
     }
 }
@@ -412,12 +422,12 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
         const int col = n0 + 32 * wn + li;
         float2 v = make_float2(alpha * cre[r], alpha * cim[r]);
         float2 *dst = Cq + (long)row * N + col;
-        if (accumulate) {
+        if (accumulate & RESULT_ACCUMULATE) {
             const float2 o = *dst;
             v.x += o.x;
             v.y += o.y;
         }
-        store_wt(dst, v);
+        store_result(dst, v, accumulate);
     }
 }
 
@@ -593,12 +603,12 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
             const int row = m0 + 8 * (r / 4) + 4 * h + (r % 4);
             float2 v = make_float2(alpha * cre[r], alpha * cim[r]);
             float2 *dst = Cq + (long)row * N + n0 + li;
-            if (accumulate) {
+            if (accumulate & RESULT_ACCUMULATE) {
                 const float2 o = *dst;
                 v.x += o.x;
                 v.y += o.y;
             }
-            store_wt(dst, v);
+            store_result(dst, v, accumulate);
         }
     } else {
         // add the SK partial accumulators of a block: each of its waves finalises 16/SK registers
@@ -623,12 +633,12 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
             const int row = m0 + 8 * (r / 4) + 4 * h + (r % 4);
             float2 v = make_float2(alpha * sre, alpha * sim);
             float2 *dst = Cq + (long)row * N + n0 + li;
-            if (accumulate) {
+            if (accumulate & RESULT_ACCUMULATE) {
                 const float2 o = *dst;
                 v.x += o.x;
                 v.y += o.y;
             }
-            store_wt(dst, v);
+            store_result(dst, v, accumulate);
         }
     }
 }
@@ -762,6 +772,11 @@ static Choice choose_variant(int mode, const float *A, const float *B, int n_fre
     return {V_STAGED, 0};
 }
 
+static int result_flags(int accumulate, int n_freq, int m, int n)
+{
+    return (accumulate ? RESULT_ACCUMULATE : 0) | (stream_bytes((long)n_freq * m * n * 8) ? RESULT_STREAM : 0);
+}
+
 template <int MODE>
 static hipError_t launch_mode(const float *A, const float *B, float *C, int n_freq, int m, int n,
                               int k, float alpha, int accumulate, FreqMap fm, hipStream_t s)
@@ -769,6 +784,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
     const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
     const long total = (long)n_freq * tilesM * tilesN;
     const Choice ch = choose_variant(MODE, A, B, n_freq, m, n, k);
+    accumulate = result_flags(accumulate, n_freq, m, n);
     const float2 *A2 = reinterpret_cast<const float2 *>(A), *B2 = reinterpret_cast<const float2 *>(B);
     float2 *C2 = reinterpret_cast<float2 *>(C);
     const int chunk = (int)((total + 7) / 8);
@@ -875,7 +891,7 @@ static bool make_mm_job(int mode, const MmArgs &a, int n_freq, MmJob &j)
     j.C = reinterpret_cast<float2 *>(a.C);
     j.M = a.m; j.N = a.n; j.K = a.k;
     j.alpha = a.alpha;
-    j.accumulate = a.accumulate;
+    j.accumulate = result_flags(a.accumulate, n_freq, a.m, a.n);
     j.q_direct = q_direct;
     j.direct_wgs = q_direct * (a.m / 64) * (a.n / 64);
     j.chunk_direct = (j.direct_wgs + 7) / 8;

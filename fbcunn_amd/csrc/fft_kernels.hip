@@ -622,7 +622,7 @@ static FwdJob make_job(const FwdArgs &a)
     j.vec4 = ((reinterpret_cast<uintptr_t>(a.in) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
     j.tbl_off = 0;
     j.herm = a.herm;
-    j.stream = spectrum_store_mode();
+    j.stream = spectrum_store_mode(a.planes, N);
     j.win = a.win;
     j.win.remap = window_remap_ok<S::T>(a.win, a.planes);
     return j;

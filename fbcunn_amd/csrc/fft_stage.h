@@ -126,7 +126,7 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
 }
 
 // Spectrum stores.  Kernels whose runs per frequency are whole 128-byte lines write them through
-// (store_nt.h), or non-temporally when the measurement knob says so; part-line runs rely on the L2 to join
+// (store_nt.h), or non-temporally when the spectrum outgrows the caches (kernels.h) or the measurement knob says so; part-line runs rely on the L2 to join
 // the workgroups that share a line and stay ordinary stores (written through, 6144 planes of 55 x 55 at
 // N = 64 with 64-byte runs take 45.2 instead of 43.2 us, 4096 planes at N = 128 with 32-byte runs 216
 // instead of 187 us).
@@ -150,8 +150,12 @@ __device__ __forceinline__ void with_store_mode(int mode, F &&body)
     }
 }
 
-int spectrum_stream_override();  // 1: non-temporal spectrum stores (a measurement knob); otherwise write-through
-inline int spectrum_store_mode() { return spectrum_stream_override() == 1 ? STORE_NT : STORE_WT; }
+int spectrum_stream_override();  // 1: non-temporal spectrum stores always (a measurement knob)
+inline int spectrum_store_mode(long planes, int n)
+{
+    if (spectrum_stream_override() == 1) return STORE_NT;
+    return stream_bytes(planes * (long)n * (n / 2 + 1) * 8) ? STORE_NT : STORE_WT;
+}
 
 // Raw staging for the forward transform: the chunk of nfloats contiguous floats at g goes to LDS as it
 // lies, by LDS-direct loads (global_load_lds): no staging registers, no LDS store instructions and no

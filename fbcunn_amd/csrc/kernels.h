@@ -126,7 +126,14 @@ const char *kernel_log_get();
 // 9 = hybrid of LDS-direct tiles and split blocks, 1 / 2 / 4 = register-fed kernel with that many
 // waves per block (falls back to the shape rule where the forced variant cannot run the shape).
 void cgemm_force_variant(int v);
-// -1: spectra are written through (default); 1: non-temporal stores where runs are whole lines
+// What one kernel writes for the next to read once (a spectrum, a contraction result) is written through to
+// the memory side, whose 256 MB cache keeps it, up to this size; beyond it, it would not survive until it is
+// read and is streamed with non-temporal stores.  Per training step, non-temporal always / never / above the
+// limit: 96 -> 256 planes, 24 x 24 (53 / 107 / 142 MB of spectra) 615 / 588 / 587 us; batch 64, 96 -> 256,
+// 55 x 55 (104 / 415 / 277 MB) 1.381 / 1.407 / 1.375 ms.
+constexpr long kStreamBytes = 144L << 20;
+inline bool stream_bytes(long bytes) { return bytes > kStreamBytes; }
+// -1: the rule above (default); 1: non-temporal spectrum stores always (where runs are whole lines)
 void spectrum_stream_force(int v);
 // The 64x64 tile kernel with clock counters: adds every workgroup's shader-clock and 100 MHz ticks to
 // ticks[0] and ticks[1] (m, n multiples of 64, k of 16)

@@ -179,10 +179,10 @@ int fbfc_plan_stage_kernel(const fbfc_plan *plan, int stage, char *name, size_t 
  * with that many waves per block.  A variant that cannot run a shape falls back to the shape rule. */
 int fbfc_debug_force_contraction_kernel(int variant);
 /* Measurement knob (no counterpart in the reference): how the forward transforms store their spectra,
- * for the whole process.  -1 = written through to the memory side, whose cache keeps them for the
- * contraction (default); 1 = non-temporal stores, streamed past the caches (where the kernel writes whole
- * 128-byte lines).  Alone a transform is equally fast either way; the pass that follows is not.  Results do
- * not depend on it. */
+ * for the whole process.  -1 = by size (default): a spectrum of up to 144 MB is written through to the
+ * memory side, whose cache keeps it for the contraction, a larger one is streamed past the caches with
+ * non-temporal stores; 1 = always non-temporal (where the kernel writes whole 128-byte lines).  Alone a
+ * transform is about as fast either way; the pass that follows is not.  Results do not depend on it. */
 int fbfc_debug_force_spectrum_streaming(int mode);
 /* Measurement (no counterpart in the reference): the shader clock the 64x64 tile contraction kernel
  * actually runs at.  Issues `launches` back-to-back launches of the per-frequency product with clock
