@@ -61,6 +61,9 @@ int imax(int a, int b) { return a > b ? a : b; }
 // 32-bit byte offsets: batch * tiles * planes (and out_planes * in_planes) must stay below
 // fft_max_planes(n).  Checked when the plan is made, so that an oversized layer is refused with the
 // numbers in the message instead of failing at its first pass.
+// complex buffers are read and written as 8-byte (re, im) pairs
+bool complex_aligned(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 7) == 0; }
+
 int planes_limit(int n, long batch, long tiles, long in_planes, long out_planes)
 {
     const long lim = fbfc::fft_max_planes(n);
@@ -746,6 +749,7 @@ static int fft2d_impl(const float *real, long planes, int h, int w, int pad_u, i
                       float *freq, void *stream)
 {
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!complex_aligned(freq)) return fail(FBFC_ERR_INVALID_ARGUMENT, "the complex buffer must be 8-byte aligned");
     if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
         return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
     if (planes < 1 || h < 1 || w < 1 || pad_u < 0 || pad_l < 0 || h + pad_u > fft_size ||
@@ -773,6 +777,7 @@ static int ifft2d_impl(const float *freq, long planes, int h, int w, int pad_u, 
                        float *real, const float *bias, int bias_period, void *stream)
 {
     if (real == nullptr || freq == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!complex_aligned(freq)) return fail(FBFC_ERR_INVALID_ARGUMENT, "the complex buffer must be 8-byte aligned");
     if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
         return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
     if (planes < 1 || h < 1 || w < 1 || pad_u < 0 || pad_l < 0 || h + pad_u > fft_size ||
@@ -896,6 +901,8 @@ static int transpose_mm_impl(const float *A, const float *B, float *C, int n_fre
                              float inv_norm, int conj_trans_a, int conj_trans_b, int accumulate, void *stream)
 {
     if (A == nullptr || B == nullptr || C == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!complex_aligned(A) || !complex_aligned(B) || !complex_aligned(C))
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "complex operands must be 8-byte aligned");
     if (n_freq < 1 || m < 1 || n < 1 || k < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
     if (conj_trans_a && conj_trans_b)
         return fail(FBFC_ERR_UNSUPPORTED_DIMENSION, "conjugate-transposing both operands is not supported");

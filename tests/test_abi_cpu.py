@@ -96,6 +96,18 @@ def test_debug_knob_validates_its_argument():
     assert _lib.lib().fbfc_debug_force_spectrum_streaming(-1) == _lib.OK
 
 
+def test_misaligned_complex_buffers_are_refused():
+    """Complex buffers are accessed as 8-byte (re, im) pairs: a pointer that is not 8-byte aligned is an
+    argument error, found before any launch (no GPU needed)."""
+    import ctypes
+    L = _lib.lib()
+    ok, odd = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1004)
+    assert L.fbfc_fft2d(ok, 4, 8, 8, 0, 0, 8, odd, None) == _lib.ERR_INVALID_ARGUMENT
+    assert b"aligned" in L.fbfc_last_error()
+    assert L.fbfc_ifft2d(odd, 4, 8, 8, 0, 0, 8, ok, None, 1, None) == _lib.ERR_INVALID_ARGUMENT
+    assert L.fbfc_transpose_mm(ok, odd, ok, 1, 4, 4, 4, ctypes.c_float(1.0), 0, 0, 0, None) == _lib.ERR_INVALID_ARGUMENT
+
+
 def test_scratch_size_query():
     assert _lib.lib().fbfc_bias_grad_scratch_bytes(128, 64) >= 64 * 4
     assert _lib.lib().fbfc_bias_grad_scratch_bytes(0, 64) == 0
