@@ -714,7 +714,8 @@ int fbfc_backward(fbfc_plan *p, const float *input, const float *grad_output, co
     } else if (need_w) {
         FBFC_STAGE(tm, fbfc::launch_rfft2d_pair(N, fgo, fw, s), "rfft2d(gradOutput, weight)");
     } else if (need_in) {
-        FBFC_STAGE(tm, fbfc::launch_rfft2d_pair(N, fgo, fin, s), "rfft2d(gradOutput, input)");
+        // the two passes would transform these in two launches of their own
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_each(N, fgo, fin, s), "rfft2d(gradOutput, input)");
     } else {
         FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, fgo, s), "rfft2d(gradOutput)");
     }

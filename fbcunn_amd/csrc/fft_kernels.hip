@@ -840,19 +840,21 @@ static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStr
         case 16: return launch_fwd<16, false>(a, b, s);
         case 32: return launch_fwd<32, false>(a, b, s);
         case 64: {
-            // planes of at most 16 x 16 at the origin (convolution kernels) take the variant that
-            // skips the zero inputs; a pair that holds such an operand is issued as two launches
+            // Every operand gets the kernel its own size asks for, whatever it is launched with (results must
+            // not depend on how transforms are grouped into launches):
+            //  * planes of at most 16 x 16 at the origin (convolution kernels): the variant that skips the zero
+            //    inputs, launched on its own;
+            //  * up to 8192 planes (about two rounds of 16-plane workgroups): the 8-plane kernel of
+            //    fft_large.hip, two workgroups per CU: what it loses on its half-line runs it more than gains
+            //    on balance (6144 planes of 55 x 55: 43.7 against 46.2 us);
+            //  * more planes: whole-line runs (16384 planes of 47 x 47: 107 against 112 us).
             auto small = [](const FwdArgs &x) { return x.h <= 16 && x.w <= 16 && x.padU == 0 && x.padL == 0; };
-            if (b != nullptr && (small(a) || small(*b))) {
+            auto rows = [&](const FwdArgs &x) { return small(x) || x.planes <= kSmallLaunch64; };
+            if (b != nullptr && (small(a) || small(*b) || rows(a) != rows(*b))) {
                 const hipError_t e = dispatch_fwd(N, a, nullptr, s);
                 return e != hipSuccess ? e : dispatch_fwd(N, *b, nullptr, s);
             }
-            // Launches of up to two rounds of 16-plane workgroups take the 8-plane kernel of
-            // fft_large.hip, two workgroups per CU: what it loses on its half-line runs it more than
-            // gains on balance (6144 planes of 55 x 55: 43.7 against 46.2 us); larger launches are
-            // faster with whole-line runs (16384 planes of 47 x 47: 107 against 112 us).
-            const long total = a.planes + (b != nullptr ? b->planes : 0);
-            if (small(a) || total <= kSmallLaunch64) return launch_rfft2d_large(N, a, b, s);
+            if (rows(a)) return launch_rfft2d_large(N, a, b, s);
             return launch_fwd<64, false>(a, b, s);
         }
         case 128: return launch_rfft2d_large(N, a, b, s);
@@ -890,6 +892,16 @@ hipError_t launch_rfft2d_triple(int N, const FwdArgs &a, const FwdArgs &b, const
     }
     const hipError_t e = dispatch_fwd(N, a, &b, s);
     return e != hipSuccess ? e : dispatch_fwd(N, c, nullptr, s);
+}
+
+// Two forward transforms that two different passes would each launch on its own: one grid where that runs
+// every plane through the kernel it would get alone (N <= 32, no windows, the same staging variant), two
+// launches otherwise (at N = 64 the kernel is chosen by the size of the launch).
+hipError_t launch_rfft2d_each(int N, const FwdArgs &a, const FwdArgs &b, hipStream_t s)
+{
+    if (N <= 32 && !a.win.on && !b.win.on && raw_ok(a) == raw_ok(b)) return dispatch_fwd(N, a, &b, s);
+    const hipError_t e = dispatch_fwd(N, a, nullptr, s);
+    return e != hipSuccess ? e : dispatch_fwd(N, b, nullptr, s);
 }
 
 hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s)

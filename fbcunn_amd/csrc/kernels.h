@@ -59,6 +59,8 @@ hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s);
 // backward(): its three forward transforms and its two inverse transforms as one launch each where one
 // kernel takes them all (N <= 32, no windows), as several launches otherwise; same results either way
 hipError_t launch_rfft2d_triple(int N, const FwdArgs &a, const FwdArgs &b, const FwdArgs &c, hipStream_t s);
+// two transforms that would otherwise be two launches of launch_rfft2d_one, with the same results
+hipError_t launch_rfft2d_each(int N, const FwdArgs &a, const FwdArgs &b, hipStream_t s);
 hipError_t launch_irfft2d_two(int N, const InvArgs &a, const InvArgs &b, hipStream_t s);
 
 // Largest number of planes one launch of an N x N transform takes (the kernels address a frequency

@@ -297,6 +297,17 @@ _GROUPED = [
     (64, 64, 128, 3, 13, 0, None, "cgemm_backward_kernel"),      # split blocks only + tiles and blocks
     (16, 96, 64, 3, 14, 1, None, "cgemm_"),                      # 96 planes, even sizes: whatever kernels fit
     (8, 32, 32, 9, 57, 0, None, "cgemm_"),                       # N = 64: stages of several launches
+    # partial reuse: backward() transforms fewer tensors and must still launch them the way its two passes do
+    # (at N = 64 the size of a launch picks the kernel)
+    (64, 128, 64, 3, 58, 1, "weight", "cgemm_"),
+    (32, 16, 256, 2, 32, 1, "weight", "cgemm_"),
+    (64, 128, 64, 3, 58, 1, "input", "cgemm_"),
+    (16, 32, 32, 3, 14, 1, "weight", "cgemm_"),                  # N = 16, even sizes
+    (16, 32, 32, 3, 13, 0, "output", "cgemm_"),
+    # input even-sized, gradOutput odd-sized: the two staging variants of the forward transform meet
+    (16, 32, 32, 2, 14, 0, "weight", "cgemm_"),
+    (16, 32, 32, 2, 14, 0, None, "cgemm_"),
+    (8, 16, 16, 4, 30, 0, "input", "cgemm_"),
 ]
 
 
