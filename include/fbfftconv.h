@@ -7,6 +7,10 @@
  * point returns FBFC_OK or an error code and never throws; the message for the
  * last error on the calling thread is fbfc_last_error().
  *
+ * A plan is used by one host thread at a time; different plans and the
+ * stand-alone entry points may be called from different host threads at once,
+ * each with its own stream.
+ *
  * Tensors are contiguous fp32, NCHW.  "planes" of a 4-D tensor (d0,d1,h,w) means
  * the d0*d1 flattened leading dimensions.
  *
