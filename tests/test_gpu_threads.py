@@ -1,6 +1,6 @@
 """Two host threads, each with its own layers and its own stream, call the library at the same time.  The
 library keeps its state per plan (buffers, reuse flags) and per thread (last error), and prepares its kernels
-once behind std::call_once, so what each thread computes must equal, bit for bit, what the same calls gave
+once per device under a mutex, so what each thread computes must equal, bit for bit, what the same calls gave
 before on one thread.  The reference runs one Lua thread (fbcunn/SpatialConvolutionFFT.lua has no locking);
 a C-ABI library has no such guarantee from its callers."""
 import threading
