@@ -258,6 +258,36 @@ def measure_fft_round_trip(nn, torch, synth, steps, warmup):
     return out
 
 
+def measure_fft_1d(nn, torch, steps, warmup):
+    """Batched 1-D transforms (fbfft1dHost's job, src/fft/FBFFTHost.cpp:119-131): 256 MiB of real rows
+    of each size, forward and unnormalised inverse; bytes = the rows once plus the half spectra once."""
+    out = {}
+    for n in (8, 32, 128):
+        rows = (1 << 26) // n
+        x = torch.rand(rows, n, device="cuda")
+        freq = torch.empty((rows, n // 2 + 1, 2), device="cuda")
+        back = torch.empty_like(x)
+        w = nn.FFTWrapper("fbfft")
+        rec = {"rows": rows}
+        for name, fn in (("fft", lambda: w.fft(x, freq)), ("ifft", lambda: w.ffti(back, freq))):
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            for _ in range(warmup):
+                fn()
+            ev0.record()
+            for _ in range(steps):
+                fn()
+            ev1.record()
+            torch.cuda.synchronize()
+            ms = ev0.elapsed_time(ev1) / steps
+            nbytes = 4 * rows * n + 8 * rows * (n // 2 + 1)
+            ach = nbytes / (ms * 1e-3) / 1e9
+            rec[name] = {"kernel": w.lastKernel(), "ms": ms, "bound": "hbm", "bytes": nbytes, "achieved": ach,
+                         "unit": "GB/s", "peak": HBM_PEAK_GBS, "frac": ach / HBM_PEAK_GBS}
+        out["n%d" % n] = rec
+        del x, freq, back
+    return out
+
+
 def measure_reuse_step(nn, torch, synth, steps, warmup):
     """The same training step with memoryReuseAll (bprop reuses FFT(weight), accGrad reuses
     FFT(gradOutput) and FFT(input)): 3 forward FFTs per step instead of 6."""
@@ -548,7 +578,8 @@ def main():
     if args.all_configs:
         line["other_workloads"] = {
             "tiled_convolution": measure_tiled(nn, torch, synth, args.steps, args.warmup),
-            "reference_benchmark_layers": measure_reference_list(nn, torch, synth, args.steps)}
+            "reference_benchmark_layers": measure_reference_list(nn, torch, synth, args.steps),
+            "fft_1d": measure_fft_1d(nn, torch, args.steps, args.warmup)}
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)
     print(json.dumps(line))
 

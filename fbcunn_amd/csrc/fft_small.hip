@@ -1,10 +1,20 @@
 // The transforms outside the convolution path that nn.FFTWrapper also offers with fbfft
 // (fbcunn/FFTWrapper.lua:53-132 -> src/fft/FBFFTHost.cpp:39-175): batched 1-D real<->complex FFTs
 // of sizes 2..128 (fbfft1dHost) and the 2-D sizes 2 and 4, which are below what the tiled 2-D
-// kernels are built for.  These are simple kernels: a lane holds its whole problem in registers
-// (two rows of a 1-D batch, packed as one complex sequence; one whole plane of a tiny 2-D batch)
+// kernels are built for.
+//
+// 1-D, sizes 8..128: one lane owns one row.  A workgroup takes a contiguous chunk of rows, copies
+// it with coalesced accesses into an LDS canvas (zero-padded rows, stride N + 4 floats: 16-byte
+// aligned and rotating over the banks), every lane transforms its row in registers as ONE complex
+// transform of half the length (z[m] = x[2m] + i x[2m+1], then the split into the row's half
+// spectrum), writes the result over its own canvas row, and the workgroup copies the chunk out,
+// again coalesced.  Bytes moved are the algorithmic ones: the rows once, the spectra once.
+// Sizes 2 and 4 (1-D and 2-D) are simple kernels: a lane holds its whole problem in registers
 // and talks to global memory directly.
 #include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
 
 #include "fft_regs.h"
 #include "kernels.h"
@@ -84,6 +94,253 @@ __global__ __launch_bounds__(256, (N >= 128) ? 1 : 2) void irfft1d_kernel(const 
             if (has_b) ob[i] = im[brev<N>(i)];
         }
     });
+}
+
+// ---------------------------------------------------------------------------------
+// 1-D, N >= 8: one row per lane, chunk of rows per workgroup staged through LDS
+// ---------------------------------------------------------------------------------
+template <int N>
+struct Rows1D {
+    static constexpr int M = N / 2;        // complex length of a lane's transform
+    static constexpr int NH = N / 2 + 1;   // stored frequencies of a row
+    static constexpr int S = N + 4;        // canvas row stride in floats (holds the N + 2 floats of a spectrum too)
+    static constexpr int LANES = (N <= 32) ? 256 : 8192 / N;  // rows per workgroup: at most 37 KB of LDS
+};
+
+// Rows [row0, row0 + nr) of `in` (n floats each) into canvas rows: value x[i] at column pad_l + i,
+// zeros elsewhere.  V floats per piece (4 needs n, pad_l and the chunk address to be multiples of 4
+// floats).  Column slot j of a row carries x[j] if j < n, else a zero for the column
+// (j + pad_l) mod N: the columns left of the row wrap around to the slots right of it.
+template <int N, int V>
+__device__ __forceinline__ void stage_rows_in(float *smem, const float *__restrict__ src, int nr, int n, int pad_l,
+                                              int tid)
+{
+    using G = Rows1D<N>;
+    constexpr int PPR = N / V;                 // pieces per canvas row
+    constexpr int PER_LANE = PPR;              // G::LANES rows * PPR pieces / G::LANES lanes
+    constexpr int CAP = (V == 4) ? 16 : 32;    // loads in flight per lane
+    constexpr int CHUNK = (PER_LANE < CAP) ? PER_LANE : CAP;
+    using Piece = typename std::conditional<V == 4, float4, float>::type;
+    static_for<PER_LANE / CHUNK>([&](auto cc) {
+        constexpr int c0 = decltype(cc)::value * CHUNK;
+        Piece v[CHUNK];
+        int dst[CHUNK];
+        static_for<CHUNK>([&](auto ii) {
+            constexpr int i = decltype(ii)::value;
+            const int idx = (c0 + i) * G::LANES + tid;
+            const int row = idx / PPR, col = (idx % PPR) * V;
+            const bool live = (row < nr) && (col < n);
+            int c = col + pad_l;
+            if (c >= N) c -= N;
+            dst[i] = row * G::S + c;
+            if constexpr (V == 4)
+                v[i] = live ? *reinterpret_cast<const float4 *>(src + row * n + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+            else
+                v[i] = live ? src[row * n + col] : 0.0f;
+        });
+        static_for<CHUNK>([&](auto ii) {
+            constexpr int i = decltype(ii)::value;
+            *reinterpret_cast<Piece *>(smem + dst[i]) = v[i];
+        });
+    });
+}
+
+// Canvas rows back to rows of n floats: real[row][i] = canvas[row][pad_l + i].
+template <int N, int V>
+__device__ __forceinline__ void stage_rows_out(const float *smem, float *__restrict__ dst, int nr, int n, int pad_l,
+                                               int tid)
+{
+    using G = Rows1D<N>;
+    constexpr int PPR = N / V;
+    using Piece = typename std::conditional<V == 4, float4, float>::type;
+    static_for<PPR>([&](auto ii) {
+        constexpr int i = decltype(ii)::value;
+        const int idx = i * G::LANES + tid;
+        const int row = idx / PPR, col = (idx % PPR) * V;
+        if (row < nr && col < n)
+            *reinterpret_cast<Piece *>(dst + row * n + col) =
+                *reinterpret_cast<const Piece *>(smem + row * G::S + pad_l + col);
+    });
+}
+
+// The spectra of rows [row0, row0 + nr), contiguous in global memory, into canvas rows (complex k of a
+// row at floats 2k, 2k+1).  W complex numbers per piece; 2 needs the chunk to start on 16 bytes.  All
+// loads of a lane are in flight together (up to 33 pieces of 16 bytes at N = 128): the lanes have no
+// other work to hide the latency behind.
+template <int N, int W>
+__device__ __forceinline__ void stage_spectra_in(float *smem, const float2 *__restrict__ src, int nr, int tid)
+{
+    using G = Rows1D<N>;
+    const int total = nr * G::NH;                       // complex numbers of the chunk
+    constexpr int PIECES = G::LANES * G::NH / W;        // LANES is even
+    constexpr int PER_LANE = (PIECES + G::LANES - 1) / G::LANES;
+    if constexpr (W == 2) {
+        float4 v[PER_LANE];
+        static_for<PER_LANE>([&](auto ii) {
+            constexpr int i = decltype(ii)::value;
+            const int e = 2 * (i * G::LANES + tid);
+            v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e + 1 < total) {
+                v[i] = *reinterpret_cast<const float4 *>(src + e);
+            } else if (e < total) {                     // the last number of a chunk with an odd count
+                const float2 a = src[e];
+                v[i].x = a.x;
+                v[i].y = a.y;
+            }
+        });
+        static_for<PER_LANE>([&](auto ii) {
+            constexpr int i = decltype(ii)::value;
+            const int e = 2 * (i * G::LANES + tid);
+            if (i * G::LANES + tid < PIECES) {
+                const int row = e / G::NH, k = e - row * G::NH;
+                const bool wrap = (k + 1 == G::NH);     // the second number opens the next row
+                *reinterpret_cast<float2 *>(smem + row * G::S + 2 * k) = make_float2(v[i].x, v[i].y);
+                *reinterpret_cast<float2 *>(smem + (wrap ? (row + 1) * G::S : row * G::S + 2 * k + 2)) =
+                    make_float2(v[i].z, v[i].w);
+            }
+        });
+    } else {
+        constexpr int CHUNK = (G::NH < 33) ? G::NH : 33;
+        static_for<(G::NH + CHUNK - 1) / CHUNK>([&](auto cc) {
+            constexpr int c0 = decltype(cc)::value * CHUNK;
+            constexpr int CN = (G::NH - c0 < CHUNK) ? G::NH - c0 : CHUNK;
+            float2 v[CN];
+            static_for<CN>([&](auto ii) {
+                constexpr int i = decltype(ii)::value;
+                const int idx = (c0 + i) * G::LANES + tid;
+                v[i] = (idx < total) ? src[idx] : make_float2(0.0f, 0.0f);
+            });
+            static_for<CN>([&](auto ii) {
+                constexpr int i = decltype(ii)::value;
+                const int idx = (c0 + i) * G::LANES + tid;
+                const int row = idx / G::NH, k = idx - row * G::NH;
+                *reinterpret_cast<float2 *>(smem + row * G::S + 2 * k) = v[i];
+            });
+        });
+    }
+}
+
+template <int N, int V>
+__global__ __launch_bounds__(Rows1D<N>::LANES) void rfft1d_rows_kernel(const float *__restrict__ in,
+                                                                       float2 *__restrict__ out, long rows, int n,
+                                                                       int pad_l)
+{
+    using G = Rows1D<N>;
+    constexpr int M = G::M;
+    __shared__ __attribute__((aligned(16))) float smem[G::LANES * G::S];
+    const int tid = threadIdx.x;
+    const long row0 = (long)blockIdx.x * G::LANES;
+    const long left = rows - row0;
+    const int nr = left < G::LANES ? (int)left : G::LANES;
+    stage_rows_in<N, V>(smem, in + row0 * n, nr, n, pad_l, tid);
+    __syncthreads();
+
+    // z[m] = x[2m] + i x[2m+1]
+    float re[M], im[M];
+    float *mine = smem + tid * G::S;
+    static_for<N / 4>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        const float4 p = reinterpret_cast<const float4 *>(mine)[j];
+        re[2 * j] = p.x;
+        im[2 * j] = p.y;
+        re[2 * j + 1] = p.z;
+        im[2 * j + 1] = p.w;
+    });
+    fft_inplace<M, false>(re, im);
+    // X[k] = E[k] + W^k O[k],  E[k] = (Z[k] + conj Z[M-k]) / 2,  O[k] = -i (Z[k] - conj Z[M-k]) / 2,  Z[M] = Z[0]
+    float xr[G::NH], xi[G::NH];
+    xr[0] = re[0] + im[0];
+    xi[0] = 0.0f;
+    xr[M] = re[0] - im[0];
+    xi[M] = 0.0f;
+    xr[M / 2] = re[brev<M>(M / 2)];
+    xi[M / 2] = -im[brev<M>(M / 2)];
+    static_for<M / 2 - 1>([&](auto kk) {
+        constexpr int k = decltype(kk)::value + 1;
+        const float a = re[brev<M>(k)], b = im[brev<M>(k)];
+        const float c = re[brev<M>(M - k)], d = im[brev<M>(M - k)];
+        const float t1 = a + c, t2 = b - d, t3 = b + d, t4 = c - a;
+        constexpr float wr = (float)(0.5 * cos2pi(k, N)), wi = (float)(-0.5 * sin2pi(k, N));
+        const float pr = wr * t3 - wi * t4, pi_ = wr * t4 + wi * t3;
+        xr[k] = 0.5f * t1 + pr;
+        xi[k] = 0.5f * t2 + pi_;
+        xr[M - k] = 0.5f * t1 - pr;
+        xi[M - k] = pi_ - 0.5f * t2;
+    });
+    // the spectrum over the lane's own canvas row (no other lane reads or writes it before the barrier)
+    static_for<M / 2>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        reinterpret_cast<float4 *>(mine)[j] = make_float4(xr[2 * j], xi[2 * j], xr[2 * j + 1], xi[2 * j + 1]);
+    });
+    reinterpret_cast<float2 *>(mine)[M] = make_float2(xr[M], xi[M]);
+    __syncthreads();
+
+    // the chunk's spectra are contiguous in global memory: piece idx is complex number idx of the chunk
+    float2 *dst = out + row0 * G::NH;
+    const int total = nr * G::NH;
+    static_for<G::NH>([&](auto ii) {
+        constexpr int i = decltype(ii)::value;
+        const int idx = i * G::LANES + tid;
+        const int row = idx / G::NH, k = idx - row * G::NH;
+        if (idx < total) dst[idx] = *reinterpret_cast<const float2 *>(smem + row * G::S + 2 * k);
+    });
+}
+
+// Unnormalised inverse: (rows, N/2+1) complex -> real[row][i] = y[pad_l + i], i < n.  The imaginary
+// parts of the bins 0 and N/2 of a row are not read, as in any complex-to-real transform.
+template <int N, int V, int W>
+__global__ __launch_bounds__(Rows1D<N>::LANES) void irfft1d_rows_kernel(const float2 *__restrict__ in,
+                                                                        float *__restrict__ out, long rows, int n,
+                                                                        int pad_l)
+{
+    using G = Rows1D<N>;
+    constexpr int M = G::M;
+    __shared__ __attribute__((aligned(16))) float smem[G::LANES * G::S];
+    const int tid = threadIdx.x;
+    const long row0 = (long)blockIdx.x * G::LANES;
+    const long left = rows - row0;
+    const int nr = left < G::LANES ? (int)left : G::LANES;
+    stage_spectra_in<N, W>(smem, in + row0 * G::NH, nr, tid);
+    __syncthreads();
+
+    // Z[k] = Ee[k] + i Oo[k],  Ee[k] = X[k] + conj X[M-k],  Oo[k] = exp(+2 pi i k / N) (X[k] - conj X[M-k])
+    float zr[M], zi[M];
+    float *mine = smem + tid * G::S;
+    static_for<M / 2>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        const float4 p = reinterpret_cast<const float4 *>(mine)[j];
+        zr[2 * j] = p.x;
+        zi[2 * j] = p.y;
+        zr[2 * j + 1] = p.z;
+        zi[2 * j + 1] = p.w;
+    });
+    {
+        const float x0 = zr[0], xm = reinterpret_cast<const float2 *>(mine)[M].x;
+        zr[0] = x0 + xm;
+        zi[0] = x0 - xm;
+        zr[M / 2] = 2.0f * zr[M / 2];
+        zi[M / 2] = -2.0f * zi[M / 2];
+    }
+    static_for<M / 2 - 1>([&](auto kk) {
+        constexpr int k = decltype(kk)::value + 1;
+        const float a = zr[k], b = zi[k], c = zr[M - k], d = zi[M - k];
+        const float sr = a + c, si = b - d, dr = a - c, di = b + d;
+        constexpr float vr = (float)cos2pi(k, N), vi = (float)sin2pi(k, N);
+        const float p = vr * dr - vi * di, q = vr * di + vi * dr;
+        zr[k] = sr - q;
+        zi[k] = si + p;
+        zr[M - k] = sr + q;
+        zi[M - k] = p - si;
+    });
+    fft_inplace<M, true>(zr, zi);
+    // y[2m] = Re z[m], y[2m+1] = Im z[m], over the lane's own canvas row
+    static_for<N / 4>([&](auto jj) {
+        constexpr int j = decltype(jj)::value;
+        reinterpret_cast<float4 *>(mine)[j] = make_float4(zr[brev<M>(2 * j)], zi[brev<M>(2 * j)],
+                                                          zr[brev<M>(2 * j + 1)], zi[brev<M>(2 * j + 1)]);
+    });
+    __syncthreads();
+    stage_rows_out<N, V>(smem, out + row0 * n, nr, n, pad_l, tid);
 }
 
 // ---------------------------------------------------------------------------------
@@ -181,17 +438,57 @@ __global__ __launch_bounds__(256) void irfft2d_tiny_kernel(const float2 *__restr
 // host launchers
 // ---------------------------------------------------------------------------------
 template <int N>
-static hipError_t launch1d(bool inverse, const float *in, float *out, long rows, int n, int pad_l, hipStream_t s)
+static hipError_t launch1d_tiny(bool inverse, const float *in, float *out, long rows, int n, int pad_l, hipStream_t s)
 {
     const long pairs = (rows + 1) / 2;
     const long blocks = (pairs + 255) / 256;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-    if (!inverse)
+    if (!inverse) {
         hipLaunchKernelGGL(rfft1d_kernel<N>, dim3((unsigned)blocks), dim3(256), 0, s, in,
                            reinterpret_cast<float2 *>(out), rows, n, pad_l);
-    else
+        kernel_log_add("rfft1d_kernel", blocks * 256);
+    } else {
         hipLaunchKernelGGL(irfft1d_kernel<N>, dim3((unsigned)blocks), dim3(256), 0, s,
                            reinterpret_cast<const float2 *>(in), out, rows, n, pad_l);
+        kernel_log_add("irfft1d_kernel", blocks * 256);
+    }
+    return hipGetLastError();
+}
+
+// 16-byte pieces need rows, padding and the real tensor itself to sit on 16-byte boundaries
+static bool rows_vec4(const float *real, int n, int pad_l)
+{
+    return n % 4 == 0 && pad_l % 4 == 0 && (reinterpret_cast<uintptr_t>(real) & 15) == 0;
+}
+
+template <int N>
+static hipError_t launch1d(bool inverse, const float *in, float *out, long rows, int n, int pad_l, hipStream_t s)
+{
+    using G = Rows1D<N>;
+    const long blocks = (rows + G::LANES - 1) / G::LANES;
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)blocks), block(G::LANES);
+    if (!inverse) {
+        float2 *freq = reinterpret_cast<float2 *>(out);
+        if (rows_vec4(in, n, pad_l))
+            hipLaunchKernelGGL((rfft1d_rows_kernel<N, 4>), grid, block, 0, s, in, freq, rows, n, pad_l);
+        else
+            hipLaunchKernelGGL((rfft1d_rows_kernel<N, 1>), grid, block, 0, s, in, freq, rows, n, pad_l);
+        kernel_log_add("rfft1d_rows_kernel", blocks * G::LANES);
+    } else {
+        const float2 *freq = reinterpret_cast<const float2 *>(in);
+        const bool wide = (reinterpret_cast<uintptr_t>(in) & 15) == 0;  // chunks start on even complex counts
+        const bool vec = rows_vec4(out, n, pad_l);
+        if (vec && wide)
+            hipLaunchKernelGGL((irfft1d_rows_kernel<N, 4, 2>), grid, block, 0, s, freq, out, rows, n, pad_l);
+        else if (vec)
+            hipLaunchKernelGGL((irfft1d_rows_kernel<N, 4, 1>), grid, block, 0, s, freq, out, rows, n, pad_l);
+        else if (wide)
+            hipLaunchKernelGGL((irfft1d_rows_kernel<N, 1, 2>), grid, block, 0, s, freq, out, rows, n, pad_l);
+        else
+            hipLaunchKernelGGL((irfft1d_rows_kernel<N, 1, 1>), grid, block, 0, s, freq, out, rows, n, pad_l);
+        kernel_log_add("irfft1d_rows_kernel", blocks * G::LANES);
+    }
     return hipGetLastError();
 }
 
@@ -199,8 +496,8 @@ static hipError_t dispatch1d(bool inverse, int N, const float *in, float *out, l
                              hipStream_t s)
 {
     switch (N) {
-        case 2: return launch1d<2>(inverse, in, out, rows, n, pad_l, s);
-        case 4: return launch1d<4>(inverse, in, out, rows, n, pad_l, s);
+        case 2: return launch1d_tiny<2>(inverse, in, out, rows, n, pad_l, s);
+        case 4: return launch1d_tiny<4>(inverse, in, out, rows, n, pad_l, s);
         case 8: return launch1d<8>(inverse, in, out, rows, n, pad_l, s);
         case 16: return launch1d<16>(inverse, in, out, rows, n, pad_l, s);
         case 32: return launch1d<32>(inverse, in, out, rows, n, pad_l, s);

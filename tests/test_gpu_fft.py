@@ -162,7 +162,9 @@ def test_fft_argument_errors(nn):
 # One transform dimension: the sizes and batch sizes of the reference's module test
 # (test/test_FFTModule.lua:170-193), plus padded rows.
 CASES_1D = [(n, rows, n, 0) for n in (2, 4, 8, 16, 32, 64, 128) for rows in (1, 127, 437)] + \
-           [(8, 33, 5, 2), (32, 1000, 27, 3), (128, 64, 100, 28), (16, 2, 1, 15)]
+           [(8, 33, 5, 2), (32, 1000, 27, 3), (128, 64, 100, 28), (16, 2, 1, 15)] + \
+           [(8, 5000, 4, 4), (16, 100001, 12, 4), (32, 70000, 32, 0), (32, 513, 31, 1), (64, 33333, 64, 0),
+            (64, 300, 60, 4), (64, 129, 62, 1), (128, 10001, 128, 0), (128, 129, 3, 125), (128, 65, 64, 64)]
 
 
 @pytest.mark.parametrize("n,rows,m,pl", CASES_1D)
@@ -193,6 +195,44 @@ def test_1d_forward_and_inverse(nn, oracle, n, rows, m, pl):
     wantb = full[:, pl:pl + m].astype(np.float64) * n
     assert np.isfinite(back).all()
     assert np.abs(back - wantb).max() <= 4 * TOL * np.abs(wantb).max()
+
+
+@pytest.mark.parametrize("n", [8, 32, 128])
+def test_1d_rows_that_do_not_start_on_16_bytes(nn, n):
+    """Row lengths that are multiples of four floats take 16-byte pieces only if the tensor itself starts on
+    a 16-byte boundary; a view one float into a buffer takes the 4-byte path and gives the same numbers."""
+    rows = 777
+    x = synth.uniform(500 + n, (rows, n))
+    buf = torch.zeros(rows * n + 1, device="cuda")
+    buf[1:] = dev(x).reshape(-1)
+    view = buf[1:].view(rows, n)
+    assert view.data_ptr() % 16 == 4
+    w = nn.FFTWrapper("fbfft")
+    fa = torch.empty((rows, n // 2 + 1, 2), device="cuda")
+    fb = torch.empty_like(fa)
+    w.fft(dev(x), fa)
+    w.fft(view, fb)
+    assert torch.equal(fa, fb)
+    want = np.fft.rfft(x.astype(np.float64))
+    got = host(fa)
+    assert np.abs(got[..., 0] + 1j * got[..., 1] - want).max() <= TOL * np.abs(want).max()
+    out_a = torch.empty((rows, n), device="cuda")
+    out_buf = torch.full((rows * n + 1,), float("nan"), device="cuda")
+    w.ffti(out_a, fa)
+    w.ffti(out_buf[1:].view(rows, n), fa)
+    assert torch.equal(out_a.reshape(-1), out_buf[1:])
+    assert torch.isnan(out_buf[0])
+    assert np.abs(host(out_a) / n - x).max() <= 1e-5 * np.abs(x).max()
+    # spectra that start 8 bytes into a buffer are read one complex number at a time, not two
+    fbuf = torch.zeros(fa.numel() + 2, device="cuda")
+    fbuf[2:] = fa.reshape(-1)
+    fview = fbuf[2:].view(rows, n // 2 + 1, 2)
+    assert fview.data_ptr() % 16 == 8
+    out_c = torch.empty((rows, n), device="cuda")
+    w.ffti(out_c, fview)
+    assert torch.equal(out_a, out_c)
+    w.ffti(out_buf[1:].view(rows, n), fview)
+    assert torch.equal(out_a.reshape(-1), out_buf[1:])
 
 
 def test_1d_round_trip_and_timed_mode(nn):
