@@ -410,20 +410,32 @@ def measure_spectrum_store_policy(nn, torch, synth, steps, warmup):
     return out
 
 
-def measure_copy_bandwidth(torch):
-    """A plain 256 MiB device-to-device copy: what HBM delivers to a trivial kernel on this box."""
-    a = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+def measure_copy_bandwidth(torch, floats=64 * 1024 * 1024, reps=10):
+    """A plain device-to-device copy (256 MiB by default): what HBM delivers to a trivial kernel on this box."""
+    a = torch.zeros(floats, dtype=torch.float32, device="cuda")
     b = torch.empty_like(a)
     for _ in range(3):
         b.copy_(a)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(10):
+    for _ in range(reps):
         b.copy_(a)
     e1.record()
     torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / 10
+    ms = e0.elapsed_time(e1) / reps
     return {"ms": ms, "GBps_read_plus_write": 2 * a.numel() * 4 / (ms * 1e-3) / 1e9}
+
+
+def measure_small_copies(torch):
+    """Plain copies that move as many bytes as the transform launches of the main workload (an inverse
+    transform reads 18.9 MB and writes 11.1 MB, a forward pair reads 22 MB and writes 38 MB): launches of
+    this size are as much ramp as streaming, and this is what the same box gives a trivial kernel for them."""
+    out = {}
+    for mb in (30, 60):
+        r = measure_copy_bandwidth(torch, floats=mb * 1000 * 1000 // 8, reps=50)
+        out["%dMB_moved" % mb] = {"ms": r["ms"], "GBps_read_plus_write": r["GBps_read_plus_write"],
+                                  "frac_of_hbm_peak": r["GBps_read_plus_write"] / HBM_PEAK_GBS}
+    return out
 
 
 def measure_mfma_clock(nn, torch):
@@ -567,6 +579,7 @@ def main():
     line["reuse_all_step"] = measure_reuse_step(nn, torch, synth, args.steps, args.warmup)
     line["fprop_plus_backward_step"] = measure_backward_step(nn, torch, synth, args.steps, args.warmup)
     line["copy_256MiB"] = measure_copy_bandwidth(torch)
+    line["copy_stage_sized"] = measure_small_copies(torch)
     line["mfma_clock"] = measure_mfma_clock(nn, torch)
     line["spectrum_store_policy"] = measure_spectrum_store_policy(nn, torch, synth, args.steps, args.warmup)
     if "mfma_issued_frac" in roofline:

@@ -748,14 +748,17 @@ static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s, const InvArgs
     return hipGetLastError();
 }
 
+static bool inv32_in_phases(long planes) { return planes > 512L * FftShape<32, true>::T; }
+
 template <int N, bool WIN>
 static hipError_t launch_inv(const InvArgs &a, hipStream_t s)
 {
     // N = 32: with the whole tile in LDS two workgroups share a CU, in two phases four do.  A launch
-    // of more than two rounds of workgroups is faster with the four (65536 planes of 27 x 27: 95 ->
-    // 84 us), a launch of one round with the whole tile (8192 planes of 27 x 27: 11.3 against 12.1 us).
+    // of more than one round of two workgroups per CU is faster with the four (12288 planes of
+    // 27 x 27: 20.9 -> 16.9 us, 65536 planes: 95 -> 84 us); up to one round the two are level
+    // (8192 planes: 10.9 and 11.0 us) and the whole tile stays.
     if constexpr (N == 32) {
-        if (a.planes > 2L * 512 * FftShape<N, true>::T) return launch_inv_impl<N, WIN, 2>(a, s);
+        if (inv32_in_phases(a.planes)) return launch_inv_impl<N, WIN, 2>(a, s);
     }
     return launch_inv_impl<N, WIN, 0>(a, s);
 }
@@ -822,6 +825,13 @@ hipError_t fft_prepare_device()
 // N = 64: launches of at most this many planes take the 8-plane kernels of fft_large.hip
 constexpr long kSmallLaunch64 = 8192;
 
+// N = 32 forward: the operand sizes that take the one-row-per-lane kernel (see dispatch_fwd)
+static bool fwd32_rows(long planes)
+{
+    const long k = (planes + 4095) / 4096;
+    return k <= 2 || k == 4;
+}
+
 static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s)
 {
     if (!planes_ok(N, a.planes) || (b != nullptr && !planes_ok(N, b->planes))) return hipErrorInvalidValue;
@@ -838,7 +848,22 @@ static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStr
     switch (N) {
         case 8: return launch_fwd<8, false>(a, b, s);
         case 16: return launch_fwd<16, false>(a, b, s);
-        case 32: return launch_fwd<32, false>(a, b, s);
+        case 32: {
+            // Per operand, as at N = 64 below.  The one-row-per-lane kernel of fft_large.hip (512 lanes, four
+            // workgroups per CU) against the two-rows-per-lane one (256 lanes, three per CU), both 16 planes
+            // per workgroup: what decides is how the workgroups of an operand divide over the CUs.  With
+            // k = ceil(planes / 4096) workgroups per CU: 8192 planes of 27 x 27 (k = 2) 11.3 -> 10.2 us,
+            // 16384 planes (k = 4) 23.3 -> 20.8 us, but 12288 planes (k = 3) 15.6 -> 16.6 us and 24576 planes
+            // (k = 6) 29.8 -> 32.1 us; beyond that the two are within a few per cent either way, and one kernel
+            // for all large operands keeps the operands of a pass in one launch.
+            auto rows = [](const FwdArgs &x) { return fwd32_rows(x.planes); };
+            if (b != nullptr && rows(a) != rows(*b)) {
+                const hipError_t e = dispatch_fwd(N, a, nullptr, s);
+                return e != hipSuccess ? e : dispatch_fwd(N, *b, nullptr, s);
+            }
+            if (rows(a)) return launch_rfft2d_large(N, a, b, s);
+            return launch_fwd<32, false>(a, b, s);
+        }
         case 64: {
             // Every operand gets the kernel its own size asks for, whatever it is launched with (results must
             // not depend on how transforms are grouped into launches):
@@ -886,7 +911,12 @@ hipError_t launch_rfft2d_triple(int N, const FwdArgs &a, const FwdArgs &b, const
         switch (N) {
             case 8: return launch_fwd<8, false>(a, &b, s, &c);
             case 16: return launch_fwd<16, false>(a, &b, s, &c);
-            case 32: return launch_fwd<32, false>(a, &b, s, &c);
+            case 32: {
+                const bool ra = fwd32_rows(a.planes), rb = fwd32_rows(b.planes), rc = fwd32_rows(c.planes);
+                if (ra && rb && rc) return launch_rfft2d_large(N, a, &b, s, &c);
+                if (ra || rb || rc) break;
+                return launch_fwd<32, false>(a, &b, s, &c);
+            }
             default: break;
         }
     }
@@ -895,8 +925,8 @@ hipError_t launch_rfft2d_triple(int N, const FwdArgs &a, const FwdArgs &b, const
 }
 
 // Two forward transforms that two different passes would each launch on its own: one grid where that runs
-// every plane through the kernel it would get alone (N <= 32, no windows, the same staging variant), two
-// launches otherwise (at N = 64 the kernel is chosen by the size of the launch).
+// every plane through the kernel it would get alone (N <= 32, no windows, the same staging variant; dispatch_fwd
+// splits a pair whose operands take different kernels), two launches otherwise.
 hipError_t launch_rfft2d_each(int N, const FwdArgs &a, const FwdArgs &b, hipStream_t s)
 {
     if (N <= 32 && !a.win.on && !b.win.on && raw_ok(a) == raw_ok(b)) return dispatch_fwd(N, a, &b, s);
@@ -936,8 +966,7 @@ hipError_t launch_irfft2d_two(int N, const InvArgs &a, const InvArgs &b, hipStre
             case 16: return launch_inv_impl<16, false, 0>(a, s, &b);
             case 32: {
                 // each tensor keeps the kernel it would get alone; one launch if that is the same kernel
-                const long two_rounds = 2L * 512 * FftShape<32, true>::T;
-                const bool pa = a.planes > two_rounds, pb = b.planes > two_rounds;
+                const bool pa = inv32_in_phases(a.planes), pb = inv32_in_phases(b.planes);
                 if (pa != pb) break;
                 return pa ? launch_inv_impl<32, false, 2>(a, s, &b) : launch_inv_impl<32, false, 0>(a, s, &b);
             }

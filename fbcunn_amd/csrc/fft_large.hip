@@ -102,7 +102,7 @@ __device__ __forceinline__ void store_column(const float (&re)[N / 2], const flo
 // the inputs that are known to be zero and the tile keeps NZ rows.
 template <int N, int T, int NZ, bool RAW>
 __global__ __launch_bounds__((RowShape<N, T, (NZ < N)>::THREADS), (RowShape<N, T, (NZ < N)>::MIN_WAVES)) void
-rfft2d_rows_kernel(FwdJob job0, FwdJob job1, unsigned blocks0)
+rfft2d_rows_kernel(FwdJob job0, FwdJob job1, FwdJob job2, unsigned blocks0, unsigned blocks01)
 {
     constexpr bool SMALL = NZ < N;
     using S = RowShape<N, T, SMALL>;
@@ -111,16 +111,19 @@ rfft2d_rows_kernel(FwdJob job0, FwdJob job1, unsigned blocks0)
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x;
     const unsigned v = blockIdx.x;
-    const bool second = v >= blocks0;
-    const float *__restrict__ in = second ? job1.in : job0.in;
-    float2 *__restrict__ out = second ? job1.out : job0.out;
-    const long planes = second ? job1.planes : job0.planes;
-    const int h = second ? job1.h : job0.h, w = second ? job1.w : job0.w;
-    const int padU = second ? job1.padU : job0.padU, padL = second ? job1.padL : job0.padL;
-    const int vec4 = second ? job1.vec4 : job0.vec4;
-    const int herm = second ? job1.herm : job0.herm;
-    const int stream = second ? job1.stream : job0.stream;
-    const long x0 = plane_group<T, S::G>(v - (second ? blocks0 : 0u)) * T;
+    // up to three tensors per launch: workgroups [0, blocks0) work on job 0, [blocks0, blocks01) on
+    // job 1, the rest on job 2
+    const bool second = v >= blocks0, third = v >= blocks01;
+    const FwdJob &job = third ? job2 : (second ? job1 : job0);
+    const float *__restrict__ in = job.in;
+    float2 *__restrict__ out = job.out;
+    const long planes = job.planes;
+    const int h = job.h, w = job.w;
+    const int padU = job.padU, padL = job.padL;
+    const int vec4 = job.vec4;
+    const int herm = job.herm;
+    const int stream = job.stream;
+    const long x0 = plane_group<T, S::G>(v - (third ? blocks01 : (second ? blocks0 : 0u))) * T;
     if (x0 >= planes) return;
     const int np = (int)((planes - x0 < (long)T) ? (planes - x0) : (long)T);
     const int hw = h * w;
@@ -503,7 +506,8 @@ static FwdJob make_rows_job(const FwdArgs &a)
 }
 
 template <int N, int T, int NZ, bool RAW>
-static hipError_t launch_fwd_rows(const FwdArgs &a, const FwdArgs *second, hipStream_t s)
+static hipError_t launch_fwd_rows(const FwdArgs &a, const FwdArgs *second, hipStream_t s,
+                                  const FwdArgs *third = nullptr)
 {
     constexpr bool SMALL = NZ < N;
     using S = RowShape<N, T, SMALL>;
@@ -511,12 +515,19 @@ static hipError_t launch_fwd_rows(const FwdArgs &a, const FwdArgs *second, hipSt
     const long blocks0 = plane_group_blocks<T, S::G>(a.planes);
     long blocks = blocks0;
     FwdJob j0 = make_rows_job<N, T, SMALL>(a);
-    FwdJob j1 = j0;
+    FwdJob j1 = j0, j2 = j0;
     if (second != nullptr) {
         const size_t lds1 = rows_lds_bytes<N, T, SMALL>(second->h, second->w);
         if (lds1 > lds) lds = lds1;
         blocks += plane_group_blocks<T, S::G>(second->planes);
         j1 = make_rows_job<N, T, SMALL>(*second);
+    }
+    const long blocks01 = blocks;
+    if (third != nullptr) {
+        const size_t lds2 = rows_lds_bytes<N, T, SMALL>(third->h, third->w);
+        if (lds2 > lds) lds = lds2;
+        blocks += plane_group_blocks<T, S::G>(third->planes);
+        j2 = make_rows_job<N, T, SMALL>(*third);
     }
     if (blocks > 0x7fffffffL || lds > 160 * 1024) return hipErrorInvalidValue;
     {
@@ -525,7 +536,7 @@ static hipError_t launch_fwd_rows(const FwdArgs &a, const FwdArgs *second, hipSt
         kernel_log_add(name, blocks * S::THREADS);
     }
     hipLaunchKernelGGL((rfft2d_rows_kernel<N, T, NZ, RAW>), dim3((unsigned)blocks), dim3(S::THREADS), lds, s, j0, j1,
-                       (unsigned)blocks0);
+                       j2, (unsigned)blocks0, (unsigned)blocks01);
     return hipGetLastError();
 }
 
@@ -567,9 +578,14 @@ static hipError_t launch_fwd64(const FwdArgs &a, const FwdArgs *b, hipStream_t s
     return raw ? launch_fwd_rows<64, 8, 64, true>(a, b, s) : launch_fwd_rows<64, 8, 64, false>(a, b, s);
 }
 
-hipError_t launch_rfft2d_large(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s)
+hipError_t launch_rfft2d_large(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s, const FwdArgs *c)
 {
-    if (a.win.on || (b != nullptr && b->win.on)) return hipErrorInvalidValue;
+    if (a.win.on || (b != nullptr && b->win.on) || (c != nullptr && (b == nullptr || c->win.on || N != 32)))
+        return hipErrorInvalidValue;
+    if (N == 32) {
+        const bool raw = raw_ok(a) && (b == nullptr || raw_ok(*b)) && (c == nullptr || raw_ok(*c));
+        return raw ? launch_fwd_rows<32, 16, 32, true>(a, b, s, c) : launch_fwd_rows<32, 16, 32, false>(a, b, s, c);
+    }
     if (N == 64) return launch_fwd64(a, b, s);
     if (N == 128) return launch_fwd_rows<128, 4, 128, false>(a, b, s);
     return hipErrorInvalidValue;

@@ -71,7 +71,7 @@ long fft_max_planes(int N);
 hipError_t fft_prepare_device();
 
 // fft_large.hip: the transforms of size 64 and 128 (plain operands; no windows)
-hipError_t launch_rfft2d_large(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s);
+hipError_t launch_rfft2d_large(int N, const FwdArgs &a, const FwdArgs *b, hipStream_t s, const FwdArgs *c = nullptr);
 hipError_t launch_irfft2d_large(int N, const InvArgs &a, hipStream_t s);
 hipError_t fft_large_prepare_device();
 

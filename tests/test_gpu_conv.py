@@ -308,6 +308,13 @@ _GROUPED = [
     (16, 32, 32, 2, 14, 0, "weight", "cgemm_"),
     (16, 32, 32, 2, 14, 0, None, "cgemm_"),
     (8, 16, 16, 4, 30, 0, "input", "cgemm_"),
+    # N = 32: the forward kernel is picked per operand by its plane count (12288 planes of gradOutput take the
+    # two-rows-per-lane kernel, 8192 of input and 6144 of weight the one-row-per-lane one); with partial reuse
+    # backward() transforms another subset of them than its two passes do
+    (128, 64, 96, 5, 27, 2, None, "cgemm_"),
+    (128, 64, 96, 5, 27, 2, "weight", "cgemm_"),
+    (128, 64, 96, 5, 27, 2, "input", "cgemm_"),
+    (128, 96, 64, 5, 26, 2, "output", "cgemm_"),
 ]
 
 
