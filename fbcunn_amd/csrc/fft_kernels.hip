@@ -822,8 +822,14 @@ hipError_t fft_prepare_device()
     return e;
 }
 
-// N = 64: launches of at most this many planes take the 8-plane kernels of fft_large.hip
-constexpr long kSmallLaunch64 = 8192;
+// N = 64: the operand sizes that take the 8-plane kernels of fft_large.hip (two workgroups per CU, half-line
+// runs).  Both forward kernels run 4096 planes per round of workgroups; the 8-plane one fills a last round
+// that is at most half full better (2048 planes of 55 x 55: 19.3 -> 18.7 us, 6144: 44.2 -> 42.0 us) and loses
+// on full rounds (4096: 25.6 -> 27.7 us, 8192: 49.4 -> 59.0 us, 12288: 81.6 -> 87.6 us).
+static bool fwd64_rows(long planes) { return planes <= 2048 || (planes > 4096 && planes <= 6144); }
+// The 8-plane inverse wins up to three rounds (2048 planes: 18.9 -> 15.4 us, 6144: 42.8 -> 37.1 us, 12288:
+// 72.1 -> 69.5 us) and loses from 16384 planes on (96.6 -> 103.4 us).
+static bool inv64_rows(long planes) { return planes <= 12288; }
 
 // N = 32 forward: the operand sizes that take the one-row-per-lane kernel (see dispatch_fwd)
 static bool fwd32_rows(long planes)
@@ -869,12 +875,11 @@ static hipError_t dispatch_fwd(int N, const FwdArgs &a, const FwdArgs *b, hipStr
             // not depend on how transforms are grouped into launches):
             //  * planes of at most 16 x 16 at the origin (convolution kernels): the variant that skips the zero
             //    inputs, launched on its own;
-            //  * up to 8192 planes (about two rounds of 16-plane workgroups): the 8-plane kernel of
-            //    fft_large.hip, two workgroups per CU: what it loses on its half-line runs it more than gains
-            //    on balance (6144 planes of 55 x 55: 43.7 against 46.2 us);
-            //  * more planes: whole-line runs (16384 planes of 47 x 47: 107 against 112 us).
+            //  * plane counts that leave the last round of 16-plane workgroups at most half full (fwd64_rows):
+            //    the 8-plane kernel of fft_large.hip;
+            //  * all others: whole-line runs (16384 planes of 47 x 47: 107 against 112 us).
             auto small = [](const FwdArgs &x) { return x.h <= 16 && x.w <= 16 && x.padU == 0 && x.padL == 0; };
-            auto rows = [&](const FwdArgs &x) { return small(x) || x.planes <= kSmallLaunch64; };
+            auto rows = [&](const FwdArgs &x) { return small(x) || fwd64_rows(x.planes); };
             if (b != nullptr && (small(a) || small(*b) || rows(a) != rows(*b))) {
                 const hipError_t e = dispatch_fwd(N, a, nullptr, s);
                 return e != hipSuccess ? e : dispatch_fwd(N, *b, nullptr, s);
@@ -950,7 +955,7 @@ hipError_t launch_irfft2d_args(int N, const InvArgs &a, hipStream_t s)
         case 16: return launch_inv<16, false>(a, s);
         case 32: return launch_inv<32, false>(a, s);
         case 64:
-            return (a.planes <= kSmallLaunch64 || (a.h <= 16 && a.w <= 16)) ? launch_irfft2d_large(N, a, s)
+            return (inv64_rows(a.planes) || (a.h <= 16 && a.w <= 16)) ? launch_irfft2d_large(N, a, s)
                                                                              : launch_inv<64, false>(a, s);
         case 128: return launch_irfft2d_large(N, a, s);
         default: return hipErrorInvalidValue;
