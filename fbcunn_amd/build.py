@@ -25,7 +25,12 @@ FLAGS = [
 # Per-file flags.  fft_large.hip: with common-code sinking the two role branches of the inverse kernel
 # end in one store through a pointer that selects between two register arrays, which forces both
 # into scratch memory.
-EXTRA_FLAGS = {"fft_large.hip": ["-mllvm", "-simplifycfg-sink-common=false"]}
+# The FFT files are compiled without implicit contraction of a multiply and an add into one operation (every
+# multiply-add they want is written as one): which pairs the compiler fuses can differ between two
+# instantiations of one kernel, and the staging variants of a transform must give the same bits.
+NO_CONTRACT = ["-ffp-contract=off"]
+EXTRA_FLAGS = {"fft_large.hip": ["-mllvm", "-simplifycfg-sink-common=false"] + NO_CONTRACT,
+               "fft_kernels.hip": NO_CONTRACT, "fft_small.hip": NO_CONTRACT}
 
 
 def _compile(src, report):

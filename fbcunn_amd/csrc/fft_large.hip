@@ -66,7 +66,7 @@ __device__ __forceinline__ void store_column(const float (&re)[N / 2], const flo
     if (!slot0) {
         static_for<M>([&](auto kk) {
             constexpr int k = decltype(kk)::value;
-            store_freq_run<WHOLE>(reinterpret_cast<float2 *>(obase + (2 * k + ROLE) * rowbytes + voff),
+            store_freq_at<WHOLE>(obase + (2 * k + ROLE) * rowbytes, voff,
                                   make_float2(re[brev<M>(k)], im[brev<M>(k)]));
         });
     } else {
@@ -84,13 +84,13 @@ __device__ __forceinline__ void store_column(const float (&re)[N / 2], const flo
             const float nr = re[brev<M>(k2)], ni = im[brev<M>(k2)];
             const float2 c0 = make_float2(0.5f * (zr + nr), 0.5f * (zi - ni));
             const float2 cn = make_float2(0.5f * (zi + ni), 0.5f * (nr - zr));
-            store_freq_run<WHOLE>(reinterpret_cast<float2 *>(obase + ky * rowbytes + voff), c0);
-            store_freq_run<WHOLE>(reinterpret_cast<float2 *>(obase + ky * rowbytes + vnyq), cn);
+            store_freq_at<WHOLE>(obase + ky * rowbytes, voff, c0);
+            store_freq_at<WHOLE>(obase + ky * rowbytes, vnyq, cn);
             if constexpr (ky > 0 && ky < N / 2) {
                 if (!herm) {
-                    store_freq_run<WHOLE>(reinterpret_cast<float2 *>(obase + (N - ky) * rowbytes + voff),
+                    store_freq_at<WHOLE>(obase + (N - ky) * rowbytes, voff,
                                           make_float2(c0.x, -c0.y));
-                    store_freq_run<WHOLE>(reinterpret_cast<float2 *>(obase + (N - ky) * rowbytes + vnyq),
+                    store_freq_at<WHOLE>(obase + (N - ky) * rowbytes, vnyq,
                                           make_float2(cn.x, -cn.y));
                 }
             }
@@ -219,9 +219,11 @@ rfft2d_rows_kernel(FwdJob job0, FwdJob job1, FwdJob job2, unsigned blocks0, unsi
             const float c = re[brev<M>(M - k)], d = im[brev<M>(M - k)];
             const float t1 = a + c, t2 = b - d, t3 = b + d, t4 = c - a;
             constexpr float wr = (float)(0.5 * cos2pi(k, N)), wi = (float)(-0.5 * sin2pi(k, N));
-            const float pr = wr * t3 - wi * t4, pi_ = wr * t4 + wi * t3;
-            put(std::integral_constant<int, k>{}, 0.5f * t1 + pr, 0.5f * t2 + pi_);
-            put(std::integral_constant<int, M - k>{}, 0.5f * t1 - pr, pi_ - 0.5f * t2);
+            // every multiply-add is spelt out: the file is compiled without implicit contraction, so that
+            // the instantiations of this kernel (raw / canvas staging) round alike
+            const float pr = __builtin_fmaf(wr, t3, -(wi * t4)), pi_ = __builtin_fmaf(wr, t4, wi * t3);
+            put(std::integral_constant<int, k>{}, __builtin_fmaf(0.5f, t1, pr), __builtin_fmaf(0.5f, t2, pi_));
+            put(std::integral_constant<int, M - k>{}, __builtin_fmaf(0.5f, t1, -pr), __builtin_fmaf(-0.5f, t2, pi_));
         });
     } else if (t < np && y < TROWS) {
         // a canvas row outside the plane is zero in every phase: written once, the refills below
@@ -385,8 +387,8 @@ irfft2d_rows_kernel(const float2 *__restrict__ in, float *__restrict__ out, long
                     im[p] = xr;
                 } else {
                     constexpr float vr = (float)cos2pi(k, N), vi = (float)sin2pi(k, N);
-                    re[p] = xr * vr - xi * vi;
-                    im[p] = xr * vi + xi * vr;
+                    re[p] = __builtin_fmaf(xr, vr, -(xi * vi));
+                    im[p] = __builtin_fmaf(xr, vi, xi * vr);
                 }
             });
         }
@@ -444,7 +446,7 @@ irfft2d_rows_kernel(const float2 *__restrict__ in, float *__restrict__ out, long
             const float a = zr[k], b = zi[k], c = zr[M - k], d = zi[M - k];
             const float sr = a + c, si = b - d, dr = a - c, di = b + d;
             constexpr float vr = (float)cos2pi(k, N), vi = (float)sin2pi(k, N);
-            const float p = vr * dr - vi * di, q = vr * di + vi * dr;
+            const float p = __builtin_fmaf(vr, dr, -(vi * di)), q = __builtin_fmaf(vr, di, vi * dr);
             zr[k] = sr - q;
             zi[k] = si + p;
             zr[M - k] = sr + q;

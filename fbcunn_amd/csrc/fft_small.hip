@@ -261,11 +261,13 @@ __global__ __launch_bounds__(Rows1D<N>::LANES) void rfft1d_rows_kernel(const flo
         const float c = re[brev<M>(M - k)], d = im[brev<M>(M - k)];
         const float t1 = a + c, t2 = b - d, t3 = b + d, t4 = c - a;
         constexpr float wr = (float)(0.5 * cos2pi(k, N)), wi = (float)(-0.5 * sin2pi(k, N));
-        const float pr = wr * t3 - wi * t4, pi_ = wr * t4 + wi * t3;
-        xr[k] = 0.5f * t1 + pr;
-        xi[k] = 0.5f * t2 + pi_;
-        xr[M - k] = 0.5f * t1 - pr;
-        xi[M - k] = pi_ - 0.5f * t2;
+        // every multiply-add is spelt out (the file is compiled without implicit contraction: the 16-byte
+        // and 4-byte staging variants of a kernel must round alike)
+        const float pr = __builtin_fmaf(wr, t3, -(wi * t4)), pi_ = __builtin_fmaf(wr, t4, wi * t3);
+        xr[k] = __builtin_fmaf(0.5f, t1, pr);
+        xi[k] = __builtin_fmaf(0.5f, t2, pi_);
+        xr[M - k] = __builtin_fmaf(0.5f, t1, -pr);
+        xi[M - k] = __builtin_fmaf(-0.5f, t2, pi_);
     });
     // the spectrum over the lane's own canvas row (no other lane reads or writes it before the barrier)
     static_for<M / 2>([&](auto jj) {
@@ -326,7 +328,7 @@ __global__ __launch_bounds__(Rows1D<N>::LANES) void irfft1d_rows_kernel(const fl
         const float a = zr[k], b = zi[k], c = zr[M - k], d = zi[M - k];
         const float sr = a + c, si = b - d, dr = a - c, di = b + d;
         constexpr float vr = (float)cos2pi(k, N), vi = (float)sin2pi(k, N);
-        const float p = vr * dr - vi * di, q = vr * di + vi * dr;
+        const float p = __builtin_fmaf(vr, dr, -(vi * di)), q = __builtin_fmaf(vr, di, vi * dr);
         zr[k] = sr - q;
         zi[k] = si + p;
         zr[M - k] = sr + q;

@@ -138,6 +138,25 @@ __device__ __forceinline__ void store_freq_run(float2 *p, const float2 &v)
     else if constexpr (MODE == STORE_WT) store_wt(p, v);
     else *p = v;
 }
+// One complex value to byte offset voff of a frequency row.  The row's address is uniform: it goes into a
+// buffer resource (scalar registers, two scalar additions per row) and the lane offset is the store's 32-bit
+// vector offset, so a store costs no vector address arithmetic (as a global store to row + voff every one
+// of the N stores of a lane carried a 64-bit vector addition).  The cache policy bits are those of
+// store_freq_run: sc1 (write-through) = 16, nt = 2.
+template <int MODE>
+__device__ __forceinline__ void store_freq_at(char *rowbase, unsigned voff, const float2 &v)
+{
+    if constexpr (MODE == STORE_ORDINARY) {
+        // part-line runs: the plain global store (as buffer stores the same runs were 8 % slower)
+        *reinterpret_cast<float2 *>(rowbase + voff) = v;
+        return;
+    }
+    typedef float fx2 __attribute__((ext_vector_type(2)));
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(rowbase, 0, -1, 0x00020000);
+    const fx2 t = {v.x, v.y};
+    constexpr int aux = (MODE == STORE_NT) ? 2 : (MODE == STORE_WT) ? 16 : 0;
+    __builtin_amdgcn_raw_buffer_store_b64(t, rsrc, (int)voff, 0, aux);
+}
 // calls body(integral_constant<int, mode>) with the run-time mode as a compile-time one
 template <bool WHOLE_LINES, class F>
 __device__ __forceinline__ void with_store_mode(int mode, F &&body)
