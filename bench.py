@@ -359,8 +359,19 @@ def measure_backward_step(nn, torch, synth, steps, warmup):
     ms = time_loop(torch, step, steps, warmup)
     ms_b = time_loop(torch, lambda: net.backward(x, g, 1.0), steps, warmup)
     net.cleanupBuffers()
-    return {"ms_per_step": ms, "ms_backward": ms_b, "steps": steps,
-            "effective_tflops": 3 * 2.0 * B * F * P * o * o * k * k / (ms * 1e-3) / 1e12}
+    # the same with memoryReuseAll: backward() then transforms gradOutput only (3 forward transforms per step)
+    wstd, seed = cfg[7], cfg[8]
+    keep = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad, "all")
+    keep.weight.copy_(torch.from_numpy(synth.normal(seed, (F, P, k, k), 0.0, wstd, stream=1)).cuda())
+    keep.bias.zero_()
+    def step_keep():
+        keep.updateOutput(x)
+        keep.backward(x, g, 1.0)
+    ms_k = time_loop(torch, step_keep, steps, warmup)
+    keep.cleanupBuffers()
+    flop = 3 * 2.0 * B * F * P * o * o * k * k
+    return {"ms_per_step": ms, "ms_backward": ms_b, "steps": steps, "effective_tflops": flop / (ms * 1e-3) / 1e12,
+            "ms_per_step_reuse_all": ms_k, "effective_tflops_reuse_all": flop / (ms_k * 1e-3) / 1e12}
 
 
 def measure_reference_list(nn, torch, synth, steps):
