@@ -250,8 +250,10 @@ __global__ __launch_bounds__(256) void cgemm_freq_kernel(const float2 *__restric
 // base + 16 l, each lane from its own global address; the tile layout in LDS is therefore
 // chosen through which 16-byte chunk each lane fetches:
 //   K-contiguous tile [64 rows][8 chunks]: one instruction = 8 rows; lane (r, c') fetches chunk
-//     c = c' ^ r of row r, so that the 16-byte reads "chunk c of 8 consecutive rows" hit 8
-//     different bank groups (XOR swizzle instead of row padding);
+//     c = c' ^ ((r >> 1) & 7) of tile row r.  A row is 32 floats, so rows r and r + 2 start on the same
+//     bank and the 16 (row parity, position) slots of 16 bytes span the 64 banks once: with the key taken
+//     from r >> 1 the 16-byte reads "chunk c of 16 consecutive rows" land on 16 different slots
+//     (keyed by r & 7 alone, rows r and r + 8 shared a slot: a two-way conflict on every read);
 //   row-contiguous tile [16 k][32 chunks]: one instruction = 2 rows, stored as they lie.
 // ---------------------------------------------------------------------------------------
 // ROWS = rows of a K-contiguous tile resp. columns of a row-contiguous one (64 or 32): ROWS / 8 blocks
@@ -268,7 +270,7 @@ __device__ __forceinline__ void lds_direct_tile(const float2 *__restrict__ Mq, i
             const float2 *g;
             if (KC) {  // rows r0 + 8 blk .. +7, complex k c0 .. c0+15
                 const int rl = lane >> 3, cs = lane & 7;
-                g = Mq + (long)(r0 + 8 * blk + rl) * ld + c0 + 2 * (cs ^ rl);
+                g = Mq + (long)(r0 + 8 * blk + rl) * ld + c0 + 2 * (cs ^ (((8 * blk + rl) >> 1) & 7));
             } else {   // 16-byte chunk c of the tile stored as it lies: k row c / (ROWS/2), complex columns 2 (c % (ROWS/2))
                 const int c = blk * 64 + lane;
                 const int kl = c / (ROWS / 2), cs = c % (ROWS / 2);
@@ -365,9 +367,9 @@ __device__ __forceinline__ void ldsdirect_body(float *lds, const float2 *__restr
     tile_barrier();
 
     const int arow = 32 * wm + li, bcol = 32 * wn + li;
-    // swizzled position of 16-byte chunk c of a K-contiguous row: 8-row block, row in block, c ^ row
-    const int a_blk = (arow >> 3) * 256 + (arow & 7) * 32, a_x = arow & 7;
-    const int b_blk = (bcol >> 3) * 256 + (bcol & 7) * 32, b_x = bcol & 7;
+    // swizzled position of 16-byte chunk c of a K-contiguous row: row * 32 floats + 4 * (c ^ key(row))
+    const int a_blk = arow * 32, a_x = (arow >> 1) & 7;
+    const int b_blk = bcol * 32, b_x = (bcol >> 1) & 7;
 
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
