@@ -15,10 +15,15 @@ oracle timed on this box's host cores and, under "configs", the same per-pass an
 per-stage records for the other stated configurations (the 8192-plane FFT round
 trip, the batch-128 updateOutput layer and the large-kernel layer).
 
-Every stage is timed twice: `ms` is the mean of STAGE_REPS back-to-back launches
-between two events (inputs warm in the caches, no event overhead), `ms_single`
-the median of single launches inside an ordinary pass, one event pair around each
-(about 2 us of event overhead included).  Roofline fractions use `ms`.  For the
+Every stage is timed three ways.  `ms_in_pass` is the median duration of the stage's
+kernel(s) inside an ordinary pass, each launch timed by the start and end of its own
+dispatch (what a profiler's kernel trace reports: operands wherever the previous
+kernel left them, no launch gap, no event overhead); `frac`, `achieved` and the
+`roofline` object use it.  `ms` is the mean of STAGE_REPS back-to-back launches of the
+same stage between two events (operands warm in the caches: `frac_warm`), `ms_single`
+one launch between two events (about 2 us of event overhead included).  `resident`
+says that the stage's whole working set fits the 256 MB memory-side cache, so that
+its "HBM" rate is in part cache bandwidth.  For the
 contraction, `algorithmic_frac` counts 8 flops per complex multiply-add and
 `mfma_issued_frac` the 6 the kernels issue (three real products per complex one):
 the second is the utilisation of the fp32 matrix pipe.  Kernel names and grids come
@@ -44,6 +49,7 @@ CONFIGS = {
 }
 MAIN = "config4_step_b128_128x128_13x13_k3_p1"
 STAGE_REPS = 10
+MALL_BYTES = 256e6           # memory-side cache: a stage whose working set fits is "resident"
 
 
 def stage_model(cfg, pass_, n, q):
@@ -76,21 +82,40 @@ def stage_model(cfg, pass_, n, q):
 TRAFFIC_PROFILE = os.path.join("profiles", "hbm_traffic_all_configs.txt")
 
 
+def csrc_digest():
+    """Short SHA-256 over the kernel sources (fbcunn_amd/csrc, sorted by name): the profile summaries
+    carry the digest of the sources they were measured on, so that a reader of a bench line can tell
+    whether a looked-up counter value belongs to the kernels that ran."""
+    import hashlib
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "fbcunn_amd", "csrc")
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".h", ".cpp")):
+            h.update(name.encode())
+            h.update(open(os.path.join(d, name), "rb").read())
+    return h.hexdigest()[:12]
+
+
 def profiled_traffic():
     """HBM bytes per launch, per (kernel, grid), from the committed rocprofv3 --pmc summary
     (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, the factors a 256 MiB device copy gives for the
-    same counters).  Empty if the file is missing."""
+    same counters), and the digest of the kernel sources the summary says it was measured on.
+    Empty if the file is missing or was measured on other sources than the ones present."""
     import re
     out = {}
     try:
         text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
     except OSError:
-        return out
+        return out, None
+    m = re.search(r"csrc_sha256=([0-9a-f]+)", text)
+    head = m.group(1) if m else None
+    if head != csrc_digest():
+        return out, head
     pat = re.compile(r"^(?:fbfc::)?(\S.*?)\s+grid=(\d+)\s+FETCH_SIZE=(\d+) KiB \(x([0-9.]+).*?WRITE_SIZE=(\d+) KiB \(x([0-9.]+)", re.M)
     for m in pat.finditer(text):
         name, grid = m.group(1).strip(), int(m.group(2))
         out[(name, grid)] = (int(m.group(3)) * float(m.group(4)) + int(m.group(5)) * float(m.group(6))) * 1024
-    return out
+    return out, head
 
 
 def split_launch(desc):
@@ -151,12 +176,20 @@ def time_each(torch, fn, steps, warmup):
 
 
 def stage_times(net, x, g, p, reps, runs):
-    """Per-stage ms of pass p with `reps` back-to-back launches per stage, and what each stage
-    launched.  Mean over `runs` passes for reps > 1, median for reps == 1."""
+    """Per-stage ms of pass p and what each stage launched.  reps > 1: `reps` back-to-back launches per
+    stage between two events, mean over `runs` passes; reps == 1: one launch between two events, median;
+    reps == -1: every launch timed by its own dispatch inside an ordinary pass, median."""
     net.timed = reps
     acc, kernels = {}, {}
     run_pass(net, x, g, p)
     for _ in range(runs):
+        if reps < 0:
+            # the timed pass is queued right behind two untimed ones, so that its kernels find the device
+            # busy, as they do in a training loop
+            net.timed = False
+            run_pass(net, x, g, p)
+            run_pass(net, x, g, p)
+            net.timed = reps
         run_pass(net, x, g, p)
         one = {}
         for s, v in net.stageTimes(x).items():
@@ -195,16 +228,19 @@ def measure_config(nn, torch, synth, name, steps, warmup, layer=None):
                  "stages": {}}
         warm, kernels = stage_times(net, x, g, p, STAGE_REPS, 3)
         single, _ = stage_times(net, x, g, p, 1, 7)
+        in_pass, _ = stage_times(net, x, g, p, -1, 15)
         model = stage_model(cfg, p, n, q)
         for s, spec in model.items():
-            ms_s = warm.get(s, 0.0)
-            if ms_s <= 0:
+            ms_w, ms_s = warm.get(s, 0.0), in_pass.get(s, 0.0)
+            if ms_w <= 0 or ms_s <= 0:
                 continue
-            st = {"kernel": kernels.get(s, ""), "ms": ms_s, "ms_single": single.get(s), "bound": spec[0]}
+            st = {"kernel": kernels.get(s, ""), "ms_in_pass": ms_s, "ms": ms_w, "ms_single": single.get(s),
+                  "bound": spec[0]}
             if spec[0] == "hbm":
                 ach = spec[1] / (ms_s * 1e-3) / 1e9
                 st.update({"bytes": spec[1], "achieved": ach, "unit": "GB/s", "peak": HBM_PEAK_GBS,
-                           "frac": ach / HBM_PEAK_GBS})
+                           "frac": ach / HBM_PEAK_GBS, "frac_warm": spec[1] / (ms_w * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                           "resident": spec[1] <= MALL_BYTES})
             else:
                 ach = spec[1] / (ms_s * 1e-3) / 1e12
                 # the kernels form a complex product from three real ones: they issue 6 of the
@@ -212,9 +248,10 @@ def measure_config(nn, torch, synth, name, steps, warmup, layer=None):
                 issued = spec[1] * 0.75
                 st.update({"flops": spec[1], "bytes": spec[2], "achieved": ach, "unit": "TFLOP/s",
                            "peak": MFMA_FP32_PEAK_TF, "frac": ach / MFMA_FP32_PEAK_TF,
+                           "frac_warm": spec[1] / (ms_w * 1e-3) / 1e12 / MFMA_FP32_PEAK_TF,
                            "algorithmic_frac": ach / MFMA_FP32_PEAK_TF, "flops_issued": issued,
                            "mfma_issued_frac": issued / (ms_s * 1e-3) / 1e12 / MFMA_FP32_PEAK_TF,
-                           "hbm_gbs": spec[2] / (ms_s * 1e-3) / 1e9})
+                           "hbm_gbs": spec[2] / (ms_s * 1e-3) / 1e9, "resident": spec[2] <= MALL_BYTES})
             entry["stages"][s] = st
         res["passes"][p] = entry
     res["fft_size"] = n
@@ -224,7 +261,8 @@ def measure_config(nn, torch, synth, name, steps, warmup, layer=None):
 
 def compact(res):
     """The per-pass / per-stage record of a configuration without the byte and flop counts."""
-    keep = ("kernel", "ms", "ms_single", "bound", "frac", "algorithmic_frac", "mfma_issued_frac")
+    keep = ("kernel", "ms_in_pass", "ms", "ms_single", "bound", "frac", "frac_warm", "resident", "algorithmic_frac",
+            "mfma_issued_frac")
     return {"ms_per_step": res["ms_per_step"], "effective_tflops": res["effective_tflops"], "fft_size": res["fft_size"],
             "passes": {p: {"ms": e["ms"], "effective_tflops": e["effective_tflops"],
                            "stages": {s: {k: st[k] for k in keep if k in st} for s, st in e["stages"].items()}}
@@ -252,9 +290,11 @@ def measure_fft_round_trip(nn, torch, synth, steps, warmup):
         ms = ev0.elapsed_time(ev1) / steps
         nbytes = 4 * planes * n * n + 8 * planes * n * (n // 2 + 1)
         ach = nbytes / (ms * 1e-3) / 1e9
+        # a stand-alone transform has no pass around it: the figure is the back-to-back one, and its 69 MB
+        # working set stays in the memory-side cache between launches
         out[name] = {"kernel": w.lastKernel(), "ms": ms, "ms_single": time_each(torch, fn, 15, 2)["median"],
                      "bound": "hbm", "bytes": nbytes, "achieved": ach, "unit": "GB/s", "peak": HBM_PEAK_GBS,
-                     "frac": ach / HBM_PEAK_GBS}
+                     "frac": ach / HBM_PEAK_GBS, "frac_warm": ach / HBM_PEAK_GBS, "resident": nbytes <= MALL_BYTES}
     return out
 
 
@@ -413,8 +453,8 @@ def measure_spectrum_store_policy(nn, torch, synth, steps, warmup):
             warm, _ = stage_times(net, x, g, "fprop", STAGE_REPS, 3)
             model = stage_model(cfg, "fprop", net._plan_for(cfg[0], cfg[3], cfg[3]).info.fft_size,
                                 net._plan_for(cfg[0], cfg[3], cfg[3]).info.n_freq)
-            out[name] = {"ms_per_step": ms_step, "fprop_fft_stage_ms": warm["fft"],
-                         "fprop_fft_stage_frac": model["fft"][1] / (warm["fft"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            out[name] = {"ms_per_step": ms_step, "fprop_fft_stage_ms_warm": warm["fft"],
+                         "fprop_fft_stage_frac_warm": model["fft"][1] / (warm["fft"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
             net.cleanupBuffers()
         finally:
             _lib.check(_lib.lib().fbfc_debug_force_spectrum_streaming(-1))
@@ -453,13 +493,14 @@ def measure_mfma_clock(nn, torch):
     """The shader clock the tile contraction kernel runs at (clock counters inside the kernel), for the main
     workload's contraction shape and for a wide one that keeps the matrix pipes busy for milliseconds.
     The published fp32 MFMA peak assumes the 2.4 GHz peak clock."""
+    from fbcunn_amd import probe   # the measurement library, not part of the shipped one
     out = {"peak_clock_mhz": 2400.0}
     for name, (Q, m, n, k, launches) in {"config4_contraction": (130, 128, 128, 128, 20),
                                          "wide_contraction_130x128x1024x1024": (130, 128, 1024, 1024, 5)}.items():
         A = torch.rand(Q, m, k, 2, device="cuda") - 0.5
         B = torch.rand(Q, n, k, 2, device="cuda") - 0.5
         C = torch.empty(Q, m, n, 2, device="cuda")
-        mhz = nn.contractionClock(0, A, B, C, launches=launches)
+        mhz = probe.contractionClock(0, A, B, C, launches=launches)
         out[name] = {"mhz": mhz, "fp32_mfma_peak_at_this_clock_tflops": MFMA_FP32_PEAK_TF * mhz / 2400.0}
         del A, B, C
     return out
@@ -549,24 +590,29 @@ def main():
             configs[name]["steps"] = n_steps
 
     main_res = measure_config(nn, torch, synth, MAIN, args.steps, args.warmup, layer=main_layer)
-    # dominant kernel of the step = the stage with the largest summed time
+    # dominant kernel of the step = the stage with the largest in-pass time
     worst, worst_ms = None, -1.0
     for p, e in main_res["passes"].items():
         for s, st in e["stages"].items():
-            if st["ms"] > worst_ms:
-                worst, worst_ms = (p, s, st), st["ms"]
+            if st["ms_in_pass"] > worst_ms:
+                worst, worst_ms = (p, s, st), st["ms_in_pass"]
     p, s, st = worst
     traffic = None
     launches = split_launch(st["kernel"])
-    table = profiled_traffic()
+    table, traffic_head = profiled_traffic()
     if len(launches) == 1 and launches[0] in table:
         traffic = table[launches[0]]
+    # achieved / frac: the kernel's duration inside an ordinary pass (its own dispatch, as a profiler's
+    # kernel trace reports it); frac_warm: 10 launches back to back with the operands warm in the caches
     roofline = {"bound": st["bound"], "achieved": st["achieved"], "peak": st["peak"], "unit": st["unit"],
-                "frac": st["frac"], "traffic": traffic,
+                "frac": st["frac"], "frac_warm": st["frac_warm"], "resident": st["resident"], "traffic": traffic,
                 "traffic_source": (TRAFFIC_PROFILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel and grid; "
                                    "not measured in this run)") if traffic is not None else None,
-                "kernel": st["kernel"], "pass": p, "stage": s, "avg_launch_ms": st["ms"],
-                "single_launch_ms": st["ms_single"]}
+                # digest of the kernel sources the profile was measured on; traffic is null when it is not
+                # the digest of the sources that ran (csrc_sha256)
+                "traffic_head": traffic_head, "csrc_sha256": csrc_digest(),
+                "kernel": st["kernel"], "pass": p, "stage": s, "avg_launch_ms": st["ms_in_pass"],
+                "warm_launch_ms": st["ms"], "single_launch_ms": st["ms_single"]}
     if "mfma_issued_frac" in st:
         # achieved / frac count the algorithmic 8 flops per complex multiply-add; the kernel issues 6 of
         # them: mfma_issued_frac is the utilisation of the fp32 matrix pipe

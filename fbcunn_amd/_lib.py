@@ -36,7 +36,8 @@ class PlanInfo(ctypes.Structure):
                 ("out_h", ctypes.c_int), ("out_w", ctypes.c_int),
                 ("input_freq_bytes", ctypes.c_size_t), ("weight_freq_bytes", ctypes.c_size_t),
                 ("output_freq_bytes", ctypes.c_size_t), ("scratch_bytes", ctypes.c_size_t),
-                ("tiles_h", ctypes.c_int), ("tiles_w", ctypes.c_int)]
+                ("tiles_h", ctypes.c_int), ("tiles_w", ctypes.c_int),
+                ("backward_freq_bytes", ctypes.c_size_t)]
 
 
 _vp, _i, _f, _l = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
@@ -56,13 +57,13 @@ SIGNATURES = {
     "fbfc_update_grad_input": (_i, [_vp, _vp, _vp, _vp, _vp]),
     "fbfc_acc_grad_parameters": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _vp]),
     "fbfc_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp]),
+    "fbfc_plan_prepare_backward": (_i, [_vp]),
     "fbfc_plan_set_reuse": (_i, [_vp, ctypes.c_uint]),
     "fbfc_plan_set_timed": (_i, [_vp, _i]),
     "fbfc_plan_stage_ms": (_i, [_vp, ctypes.POINTER(_f), _i]),
     "fbfc_plan_stage_kernel": (_i, [_vp, _i, ctypes.c_char_p, ctypes.c_size_t]),
     "fbfc_debug_force_contraction_kernel": (_i, [_i]),
     "fbfc_debug_force_spectrum_streaming": (_i, [_i]),
-    "fbfc_debug_contraction_clock": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, ctypes.POINTER(_f), _vp]),
     "fbfc_fft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp]),
     "fbfc_ifft2d": (_i, [_vp, _l, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
     "fbfc_planes_layout_workspace_bytes": (ctypes.c_size_t, [_l, _i]),

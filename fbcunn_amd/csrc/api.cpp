@@ -26,6 +26,23 @@ void kernel_log_add(const char *name, long grid_items)
 }
 const char *kernel_log_get() { return g_kernel_log.c_str(); }
 
+// Per-launch timing (kernels.h): the list of event pairs the launches of this thread draw from while a
+// pass with per-launch timing runs.
+struct LaunchEvents {
+    hipEvent_t *ev;
+    int n, used;
+};
+static thread_local LaunchEvents g_launch_events = {nullptr, 0, 0};
+bool launch_events_next(hipEvent_t *start, hipEvent_t *stop)
+{
+    LaunchEvents &l = g_launch_events;
+    if (l.ev == nullptr || l.used + 2 > l.n) return false;
+    *start = l.ev[l.used];
+    *stop = l.ev[l.used + 1];
+    l.used += 2;
+    return true;
+}
+
 }  // namespace fbfc
 
 namespace {
@@ -123,6 +140,7 @@ int plan_query(const fbfc_conv_desc *d, fbfc_plan_info *info)
     info->scratch_bytes = fbfc::bias_grad_scratch_bytes(d->batch, d->out_planes);
     info->tiles_h = 1;
     info->tiles_w = 1;
+    info->backward_freq_bytes = info->input_freq_bytes + info->weight_freq_bytes;
     return FBFC_OK;
 }
 
@@ -176,6 +194,7 @@ int plan_query_tiled(const fbfc_conv_desc *d, int tile_h, int tile_w, fbfc_plan_
     info->scratch_bytes = fbfc::bias_grad_scratch_bytes(d->batch, d->out_planes);
     info->tiles_h = ceil_div(out_h, step_h);
     info->tiles_w = ceil_div(out_w, step_w);
+    info->backward_freq_bytes = 0;  // a tiled backward() runs as its two passes
     return FBFC_OK;
 }
 
@@ -202,12 +221,12 @@ struct fbfc_plan {
     pass_geom fprop, bprop, accgrad;
     int device;
     float *in_freq, *w_freq, *out_freq, *res_freq, *scratch;
-    float *bw_gi, *bw_gw;  // result spectra of fbfc_backward's single-grid stages, made at its first call
-    bool bw_failed;
+    float *bw_gi, *bw_gw;  // result spectra of fbfc_backward's single-grid stages (fbfc_plan_prepare_backward)
     unsigned reuse;
     bool have_in, have_w, have_out;  // which forward spectra are valid in their buffer
-    int timed;
+    int timed;  // > 0: repetitions per stage between two events; < 0: every launch timed by its own dispatch
     hipEvent_t ev[FBFC_NUM_STAGES + 1];
+    hipEvent_t kev[2 * 16];  // per-launch timing: a (start, stop) pair for each of up to 16 launches of a pass
     bool ev_made;
     float stage_ms[FBFC_NUM_STAGES];
     char stage_kernel[FBFC_NUM_STAGES][160];  // what each stage of the last pass launched
@@ -221,15 +240,22 @@ struct StageTimer {
     hipStream_t s;
     int n;
     int slot[FBFC_NUM_STAGES];
+    int first_ev[FBFC_NUM_STAGES + 1];  // per-launch timing: events used before each recorded stage
     StageTimer(fbfc_plan *plan, hipStream_t stream) : p(plan), s(stream), n(0)
     {
         for (auto &name : p->stage_kernel) name[0] = 0;
         fbfc::kernel_log_clear();
         if (p->timed) {
             for (float &m : p->stage_ms) m = 0.0f;
-            (void)hipEventRecord(p->ev[0], s);
+            if (p->timed > 0) {
+                (void)hipEventRecord(p->ev[0], s);
+            } else {
+                fbfc::g_launch_events = {p->kev, (int)(sizeof p->kev / sizeof p->kev[0]), 0};
+                first_ev[0] = 0;
+            }
         }
     }
+    ~StageTimer() { fbfc::g_launch_events = {nullptr, 0, 0}; }
     // number of back-to-back launches of each stage (1 unless the plan is timed)
     int reps() const { return p->timed > 0 ? p->timed : 1; }
     // after the first of several repetitions: what it logged is the stage's launch list
@@ -245,11 +271,29 @@ struct StageTimer {
         if (!p->timed) return;
         slot[n] = stage;
         ++n;
-        (void)hipEventRecord(p->ev[n], s);
+        if (p->timed > 0) (void)hipEventRecord(p->ev[n], s);
+        else first_ev[n] = fbfc::g_launch_events.used;
     }
     int finish()
     {
         if (!p->timed) return FBFC_OK;
+        if (p->timed < 0) {
+            // every launch carried its own (start, stop) pair: a stage is the sum of its launches
+            fbfc::g_launch_events = {nullptr, 0, 0};
+            hipError_t e = hipStreamSynchronize(s);
+            if (e != hipSuccess) return fail_hip(e, "hipStreamSynchronize");
+            for (int i = 0; i < n; ++i) {
+                float sum = 0.0f;
+                for (int k = first_ev[i]; k < first_ev[i + 1]; k += 2) {
+                    float ms = 0.0f;
+                    e = hipEventElapsedTime(&ms, p->kev[k], p->kev[k + 1]);
+                    if (e != hipSuccess) return fail_hip(e, "hipEventElapsedTime");
+                    sum += ms;
+                }
+                p->stage_ms[slot[i]] = sum;
+            }
+            return FBFC_OK;
+        }
         hipError_t e = hipEventSynchronize(p->ev[n]);
         if (e != hipSuccess) return fail_hip(e, "hipEventSynchronize");
         for (int i = 0; i < n; ++i) {
@@ -412,8 +456,10 @@ int fbfc_plan_destroy(fbfc_plan *p)
     if (p->scratch) (void)hipFree(p->scratch);
     if (p->bw_gi) (void)hipFree(p->bw_gi);
     if (p->bw_gw) (void)hipFree(p->bw_gw);
-    if (p->ev_made)
+    if (p->ev_made) {
         for (hipEvent_t &ev : p->ev) (void)hipEventDestroy(ev);
+        for (hipEvent_t &ev : p->kev) (void)hipEventDestroy(ev);
+    }
     delete p;
     return FBFC_OK;
 }
@@ -452,9 +498,10 @@ int fbfc_plan_set_timed(fbfc_plan *p, int on)
     if (p == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null plan");
     if (on && !p->ev_made) {
         for (hipEvent_t &ev : p->ev) FBFC_TRY(hipEventCreate(&ev), "hipEventCreate");
+        for (hipEvent_t &ev : p->kev) FBFC_TRY(hipEventCreate(&ev), "hipEventCreate");
         p->ev_made = true;
     }
-    p->timed = on > 0 ? on : 0;
+    p->timed = on;
     return FBFC_OK;
 }
 
@@ -478,31 +525,6 @@ int fbfc_debug_force_spectrum_streaming(int mode)
 {
     if (mode != -1 && mode != 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "spectrum streaming mode must be -1 or 1");
     fbfc::spectrum_stream_force(mode);
-    return FBFC_OK;
-}
-
-int fbfc_debug_contraction_clock(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
-                                 int k, int launches, float *mhz, void *stream)
-{
-    if (A == nullptr || B == nullptr || C == nullptr || mhz == nullptr || launches < 1)
-        return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    unsigned long long *ticks = nullptr;
-    FBFC_TRY(hipMalloc(reinterpret_cast<void **>(&ticks), 2 * sizeof *ticks), "hipMalloc");
-    hipError_t e = hipSuccess;
-    // the clock settles over the run of launches: the last one is the one read
-    for (int i = 0; i < launches && e == hipSuccess; ++i) {
-        if (i == launches - 1) e = hipMemsetAsync(ticks, 0, 2 * sizeof *ticks, s);
-        if (e == hipSuccess) e = fbfc::launch_cgemm_clock_probe(mode, A, B, C, n_freq, m, n, k, ticks, s);
-    }
-    unsigned long long h[2] = {0, 0};
-    if (e == hipSuccess) e = hipMemcpyAsync(h, ticks, sizeof h, hipMemcpyDeviceToHost, s);
-    if (e == hipSuccess) e = hipStreamSynchronize(s);
-    (void)hipFree(ticks);
-    if (e == hipErrorInvalidValue)
-        return fail(FBFC_ERR_INVALID_ARGUMENT, "the clock probe takes m, n multiples of 64 and k of 16");
-    if (e != hipSuccess) return fail_hip(e, "contraction clock probe");
-    *mhz = h[1] ? (float)((double)h[0] / ((double)h[1] / 100.0)) : 0.0f;
     return FBFC_OK;
 }
 
@@ -662,21 +684,24 @@ int fbfc_acc_grad_parameters(fbfc_plan *p, const float *input, const float *grad
 }
 
 // The buffers the one-grid-per-stage backward pass writes its two product spectra to (it reads all
-// three operand spectra in one launch, so neither result may overwrite one of them).
-static bool backward_buffers(fbfc_plan *p)
+// three operand spectra in one launch, so neither result may overwrite one of them).  Made here, on the
+// plan's device, never inside a pass.
+int fbfc_plan_prepare_backward(fbfc_plan *p)
 {
-    if (p->bw_gi != nullptr && p->bw_gw != nullptr) return true;
-    if (p->bw_failed) return false;
+    if (p == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null plan");
+    if (p->tiled || (p->bw_gi != nullptr && p->bw_gw != nullptr)) return FBFC_OK;
+    int current = 0;
+    FBFC_TRY(hipGetDevice(&current), "hipGetDevice");
+    if (current != p->device) FBFC_TRY(hipSetDevice(p->device), "hipSetDevice");
     hipError_t e = hipSuccess;
     if (p->bw_gi == nullptr) e = hipMalloc(reinterpret_cast<void **>(&p->bw_gi), p->info.input_freq_bytes);
     if (e == hipSuccess && p->bw_gw == nullptr)
         e = hipMalloc(reinterpret_cast<void **>(&p->bw_gw), p->info.weight_freq_bytes);
-    if (e != hipSuccess) {
-        (void)hipGetLastError();
-        p->bw_failed = true;  // no room: the pass runs as its two halves, which need no extra buffer
-        return false;
-    }
-    return true;
+    if (e != hipSuccess) (void)hipGetLastError();
+    if (current != p->device) (void)hipSetDevice(current);
+    if (e == hipErrorOutOfMemory) return fail(FBFC_ERR_OUT_OF_MEMORY, "Not enough memory for FFT buffers");
+    if (e != hipSuccess) return fail_hip(e, "backward buffers");
+    return FBFC_OK;
 }
 
 int fbfc_backward(fbfc_plan *p, const float *input, const float *grad_output, const float *weight,
@@ -685,7 +710,7 @@ int fbfc_backward(fbfc_plan *p, const float *input, const float *grad_output, co
     if (p == nullptr || input == nullptr || grad_output == nullptr || weight == nullptr ||
         grad_input == nullptr || grad_weight == nullptr)
         return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
-    if (p->tiled || !backward_buffers(p)) {
+    if (p->tiled || p->bw_gi == nullptr || p->bw_gw == nullptr) {
         const int rc = fbfc_update_grad_input(p, grad_output, weight, grad_input, stream);
         if (rc != FBFC_OK) return rc;
         // updateGradInput leaves FFT(gradOutput) in the plan (have_out; not for tiled plans, whose two
@@ -817,6 +842,8 @@ int fbfc_fft2d_planes(const float *real, long planes, int h, int w, int pad_u, i
                       float *freq_planes, float *workspace, void *stream)
 {
     if (freq_planes == nullptr || workspace == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!complex_aligned(freq_planes))
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "the complex buffer must be 8-byte aligned");
     fbfc::kernel_log_clear();
     const int rc = fft2d_impl(real, planes, h, w, pad_u, pad_l, fft_size, workspace, stream);
     if (rc != FBFC_OK) return rc;
@@ -831,9 +858,13 @@ int fbfc_ifft2d_planes(const float *freq_planes, long planes, int h, int w, int 
 {
     if (freq_planes == nullptr || workspace == nullptr || real == nullptr)
         return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
+    if (!complex_aligned(freq_planes) || !complex_aligned(workspace))
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "the complex buffer must be 8-byte aligned");
     if (!fft_size_ok(fft_size) && !fft_size_tiny(fft_size))
         return fail(FBFC_ERR_UNSUPPORTED_SIZE, "FBFFT error: unsupported size");
-    if (planes < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    // everything the inverse transform would refuse is refused before the conversion is launched
+    if (planes < 1 || h < 1 || w < 1 || pad_u < 0 || pad_l < 0 || h + pad_u > fft_size || w + pad_l > fft_size)
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "plane plus padding must fit the FFT size");
     fbfc::kernel_log_clear();
     FBFC_TRY(fbfc::launch_planes_to_freq(freq_planes, workspace, planes, fft_size * (fft_size / 2 + 1), fft_size,
                                          planes_layout_mode(fft_size), static_cast<hipStream_t>(stream)),
@@ -857,6 +888,10 @@ int fbfc_transpose_mm_planes(const float *A, const float *B, float *C, int n_fre
     if (A == nullptr || B == nullptr || C == nullptr || workspace == nullptr)
         return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     if (n_freq < 1 || m < 1 || n < 1 || k < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "sizes must be positive");
+    if (!complex_aligned(A) || !complex_aligned(B) || !complex_aligned(C) || !complex_aligned(workspace))
+        return fail(FBFC_ERR_INVALID_ARGUMENT, "complex operands must be 8-byte aligned");
+    if (conj_trans_a && conj_trans_b)
+        return fail(FBFC_ERR_UNSUPPORTED_DIMENSION, "conjugate-transposing both operands is not supported");
     hipStream_t s = static_cast<hipStream_t>(stream);
     float *wa = workspace;
     float *wb = wa + (size_t)n_freq * m * k * 2;

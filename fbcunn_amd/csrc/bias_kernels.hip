@@ -76,7 +76,7 @@ hipError_t launch_bias_grad_dc(const float *freq, float *grad_bias, float scale,
                                hipStream_t s)
 {
     BiasGradJob job = {reinterpret_cast<const float2 *>(freq), grad_bias, scale, batch, planes};
-    hipLaunchKernelGGL(bias_grad_dc_kernel, dim3(bias_grad_dc_blocks(planes)), dim3(256), 0, s, job);
+    FBFC_LAUNCH(bias_grad_dc_kernel, dim3(bias_grad_dc_blocks(planes)), dim3(256), 0, s, job);
     return hipGetLastError();
 }
 
@@ -90,7 +90,7 @@ size_t bias_grad_scratch_bytes(int batch, int planes)
 hipError_t launch_bias_add(float *out, const float *bias, int batch, int planes, int hw,
                            hipStream_t s)
 {
-    hipLaunchKernelGGL(bias_add_kernel, dim3((unsigned)((long)batch * planes)), dim3(256), 0, s, out,
+    FBFC_LAUNCH(bias_add_kernel, dim3((unsigned)((long)batch * planes)), dim3(256), 0, s, out,
                        bias, planes, hw);
     return hipGetLastError();
 }
@@ -99,11 +99,11 @@ hipError_t launch_bias_grad(const float *grad_out, float *grad_bias, float scale
                             int planes, int hw, float *scratch, hipStream_t s)
 {
     const int split = split_for(batch);
-    hipLaunchKernelGGL(bias_grad_partial_kernel, dim3(planes, split), dim3(256), 0, s, grad_out,
+    FBFC_LAUNCH(bias_grad_partial_kernel, dim3(planes, split), dim3(256), 0, s, grad_out,
                        scratch, batch, planes, hw, split);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((planes + 255) / 256), dim3(256), 0, s, scratch,
+    FBFC_LAUNCH(bias_grad_final_kernel, dim3((planes + 255) / 256), dim3(256), 0, s, scratch,
                        grad_bias, scale, planes, split);
     return hipGetLastError();
 }
@@ -170,7 +170,7 @@ hipError_t launch_bias_add_strided(float *out, const float *bias, int batch, int
                                    long sb, long sf, long sh, long sw, long bias_stride, hipStream_t s)
 {
     const Strides4 st = {sb, sf, sh, sw};
-    hipLaunchKernelGGL(bias_add_strided_kernel, dim3((unsigned)((long)batch * planes)), dim3(256), 0, s, out,
+    FBFC_LAUNCH(bias_add_strided_kernel, dim3((unsigned)((long)batch * planes)), dim3(256), 0, s, out,
                        bias, planes, h, w, st, bias_stride);
     return hipGetLastError();
 }
@@ -181,11 +181,11 @@ hipError_t launch_bias_grad_strided(const float *grad_out, float *grad_bias, flo
 {
     const Strides4 st = {sb, sf, sh, sw};
     const int split = split_for(batch);
-    hipLaunchKernelGGL(bias_grad_partial_strided_kernel, dim3(planes, split), dim3(256), 0, s, grad_out,
+    FBFC_LAUNCH(bias_grad_partial_strided_kernel, dim3(planes, split), dim3(256), 0, s, grad_out,
                        scratch, batch, h, w, st, split);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(bias_grad_final_strided_kernel, dim3((planes + 255) / 256), dim3(256), 0, s, scratch,
+    FBFC_LAUNCH(bias_grad_final_strided_kernel, dim3((planes + 255) / 256), dim3(256), 0, s, scratch,
                        grad_bias, scale, planes, split, bias_stride);
     return hipGetLastError();
 }

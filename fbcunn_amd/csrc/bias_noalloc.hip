@@ -9,6 +9,7 @@
 // device with that device current, and that pointer is what the kernels get.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "kernels.h"
@@ -27,7 +28,7 @@ int bias_grad_noalloc_max_planes() { return kNoAllocMaxPlanes; }
 static float *scratch_on_current_device(hipError_t *err)
 {
     static std::mutex mu;
-    static float *ptr[64] = {};
+    static std::atomic<float *> ptr[64] = {};
     int dev = 0;
     *err = hipGetDevice(&dev);
     if (*err != hipSuccess) return nullptr;
@@ -35,14 +36,19 @@ static float *scratch_on_current_device(hipError_t *err)
         *err = hipErrorInvalidDevice;
         return nullptr;
     }
+    // after the first call on a device the pointer is read without the lock
+    float *known = ptr[dev].load(std::memory_order_acquire);
+    if (known != nullptr) return known;
     std::lock_guard<std::mutex> lock(mu);
-    if (ptr[dev] == nullptr) {
+    known = ptr[dev].load(std::memory_order_relaxed);
+    if (known == nullptr) {
         void *p = nullptr;
         *err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (*err != hipSuccess) return nullptr;
-        ptr[dev] = static_cast<float *>(p);
+        known = static_cast<float *>(p);
+        ptr[dev].store(known, std::memory_order_release);
     }
-    return ptr[dev];
+    return known;
 }
 
 hipError_t bias_grad_noalloc_prepare()

@@ -451,6 +451,7 @@ __global__ __launch_bounds__(128 * WN) void cgemm_ldsdirect_kernel(const float2 
     ldsdirect_body<MODE, WN>(lds, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, wg, 0, fm);
 }
 
+#ifdef FBFC_PROBES  // only in the measurement library (libfbfftconv_probe.so), never in the shipped one
 // Measurement variant of the 64x64 tile kernel: each workgroup also adds the shader-clock ticks
 // (s_memtime) and the 100 MHz ticks (s_memrealtime) it lived for to ticks[0] and ticks[1]; their ratio
 // is the clock the kernel actually ran at.  Under sustained fp32 MFMA load the chip settles well below its
@@ -473,6 +474,7 @@ __global__ __launch_bounds__(256) void cgemm_ldsdirect_clock_kernel(const float2
         atomicAdd(ticks + 1, (unsigned long long)(wall_clock64() - w0));
     }
 }
+#endif  // FBFC_PROBES
 
 // ---------------------------------------------------------------------------------------
 // Split-K kernel for small problems (few 64x64 tiles per CU).
@@ -708,7 +710,7 @@ static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_
     const long wgs = (tot32 * SK + 3) / 4;
     const int chunk = (int)((wgs + 7) / 8);
     note_kernel("cgemm_splitk_kernel", MODE, SK, (long)chunk * 8 * 256);
-    hipLaunchKernelGGL((cgemm_splitk_kernel<MODE, SK>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
+    FBFC_LAUNCH((cgemm_splitk_kernel<MODE, SK>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
                        reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tm, tn, (int)tot32,
                        (int)wgs, chunk, fm);
@@ -797,7 +799,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
             const int split_tiles = (n_freq - ch.q_direct) * (m / 32) * (n / 32);  // one workgroup per 32x32 block
             const int chunk_direct = (direct_wgs + 7) / 8, chunk_split = (split_tiles + 7) / 8;
             note_kernel("cgemm_hybrid_kernel", MODE, -1, (long)(chunk_direct + chunk_split) * 8 * 256);
-            hipLaunchKernelGGL(cgemm_hybrid_kernel<MODE>, dim3((unsigned)((chunk_direct + chunk_split) * 8)),
+            FBFC_LAUNCH(cgemm_hybrid_kernel<MODE>, dim3((unsigned)((chunk_direct + chunk_split) * 8)),
                                dim3(256), 0, s, A2, B2, C2, m, n, k, alpha, accumulate, ch.q_direct, direct_wgs,
                                chunk_direct, split_tiles, split_tiles, chunk_split, fm);
             return hipGetLastError();
@@ -807,7 +809,7 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
             const long tot = (long)n_freq * tilesM * t32;
             const int c32 = (int)((tot + 7) / 8);
             note_kernel("cgemm_ldsdirect_kernel", MODE, 1, (long)c32 * 8 * 128);
-            hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 1>), dim3((unsigned)(c32 * 8)), dim3(128), 0, s, A2, B2,
+            FBFC_LAUNCH((cgemm_ldsdirect_kernel<MODE, 1>), dim3((unsigned)(c32 * 8)), dim3(128), 0, s, A2, B2,
                                C2, m, n, k, alpha, accumulate, tilesM, t32, (int)tot, c32, fm);
             return hipGetLastError();
         }
@@ -816,12 +818,12 @@ static hipError_t launch_mode(const float *A, const float *B, float *C, int n_fr
         case V_SPLIT1: return launch_splitk<MODE, 1>(A, B, C, n_freq, m, n, k, alpha, accumulate, fm, s);
         case V_TILES:
             note_kernel("cgemm_ldsdirect_kernel", MODE, 2, (long)chunk * 8 * 256);
-            hipLaunchKernelGGL((cgemm_ldsdirect_kernel<MODE, 2>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s, A2,
+            FBFC_LAUNCH((cgemm_ldsdirect_kernel<MODE, 2>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s, A2,
                                B2, C2, m, n, k, alpha, accumulate, tilesM, tilesN, (int)total, chunk, fm);
             return hipGetLastError();
         case V_STAGED:
             note_kernel("cgemm_freq_kernel", MODE, -1, (long)chunk * 8 * 256);
-            hipLaunchKernelGGL(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s, A2, B2, C2, m,
+            FBFC_LAUNCH(cgemm_freq_kernel<MODE>, dim3((unsigned)(chunk * 8)), dim3(256), 0, s, A2, B2, C2, m,
                                n, k, alpha, accumulate, tilesM, tilesN, (int)total, chunk, fm);
             return hipGetLastError();
         default: return hipErrorInvalidValue;
@@ -909,7 +911,7 @@ hipError_t launch_cgemm_backward(const MmArgs &gi, const MmArgs &gw, int n_freq,
         const long chunks = (long)j1.chunk_direct + j2.chunk_direct + j1.chunk_split + j2.chunk_split;
         if (chunks * 8 < 0x7fffff00L) {
             kernel_log_add("cgemm_backward_kernel", chunks * 8 * 256);
-            hipLaunchKernelGGL(cgemm_backward_kernel, dim3((unsigned)(chunks * 8)), dim3(256), 0, s, j1, j2, fm);
+            FBFC_LAUNCH(cgemm_backward_kernel, dim3((unsigned)(chunks * 8)), dim3(256), 0, s, j1, j2, fm);
             return hipGetLastError();
         }
     }
@@ -918,6 +920,7 @@ hipError_t launch_cgemm_backward(const MmArgs &gi, const MmArgs &gw, int n_freq,
     return launch_mode<2>(gw.A, gw.B, gw.C, n_freq, gw.m, gw.n, gw.k, gw.alpha, gw.accumulate, fm, s);
 }
 
+#ifdef FBFC_PROBES
 hipError_t launch_cgemm_clock_probe(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
                                     int k, unsigned long long *ticks, hipStream_t s)
 {
@@ -932,12 +935,13 @@ hipError_t launch_cgemm_clock_probe(int mode, const float *A, const float *B, fl
     float2 *C2 = reinterpret_cast<float2 *>(C);
     const dim3 grid((unsigned)(chunk * 8)), block(256);
     switch (mode) {
-        case 0: hipLaunchKernelGGL(cgemm_ldsdirect_clock_kernel<0>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
-        case 1: hipLaunchKernelGGL(cgemm_ldsdirect_clock_kernel<1>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
-        default: hipLaunchKernelGGL(cgemm_ldsdirect_clock_kernel<2>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
+        case 0: FBFC_LAUNCH(cgemm_ldsdirect_clock_kernel<0>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
+        case 1: FBFC_LAUNCH(cgemm_ldsdirect_clock_kernel<1>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
+        default: FBFC_LAUNCH(cgemm_ldsdirect_clock_kernel<2>, grid, block, 0, s, A2, B2, C2, m, n, k, 1.0f, tilesM, tilesN, (int)total, chunk, ticks); break;
     }
     return hipGetLastError();
 }
+#endif  // FBFC_PROBES
 
 hipError_t launch_cgemm_freq_map(int mode, const float *A, const float *B, float *C, int n_freq, FreqMap fm,
                                  int m, int n, int k, float alpha, int accumulate, hipStream_t s)

@@ -122,7 +122,7 @@ hipError_t launch_direct_fprop(const int *desc, const float *in, const float *w,
     const DirectGeom g = geom(desc);
     const long total = (long)g.B * g.F * g.oH * g.oW;
     kernel_log_add("direct_fprop_kernel", (long)grid_for(total) * 256);
-    hipLaunchKernelGGL(direct_fprop_kernel, dim3(grid_for(total)), dim3(256), 0, s, in, w, bias, out, g);
+    FBFC_LAUNCH(direct_fprop_kernel, dim3(grid_for(total)), dim3(256), 0, s, in, w, bias, out, g);
     return hipGetLastError();
 }
 
@@ -131,7 +131,7 @@ hipError_t launch_direct_bprop(const int *desc, const float *go, const float *w,
     const DirectGeom g = geom(desc);
     const long total = (long)g.B * g.P * g.H * g.W;
     kernel_log_add("direct_bprop_kernel", (long)grid_for(total) * 256);
-    hipLaunchKernelGGL(direct_bprop_kernel, dim3(grid_for(total)), dim3(256), 0, s, go, w, gi, g);
+    FBFC_LAUNCH(direct_bprop_kernel, dim3(grid_for(total)), dim3(256), 0, s, go, w, gi, g);
     return hipGetLastError();
 }
 
@@ -142,7 +142,7 @@ hipError_t launch_direct_accgrad(const int *desc, const float *in, const float *
     const long total = (long)g.F * g.P * g.kH * g.kW;
     if (total > 0x7fffffffL) return hipErrorInvalidValue;
     kernel_log_add("direct_accgrad_kernel", total * 256);
-    hipLaunchKernelGGL(direct_accgrad_kernel, dim3((unsigned)total), dim3(256), 0, s, in, go, gw, scale, g);
+    FBFC_LAUNCH(direct_accgrad_kernel, dim3((unsigned)total), dim3(256), 0, s, in, go, gw, scale, g);
     return hipGetLastError();
 }
 

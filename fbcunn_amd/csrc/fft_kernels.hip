@@ -671,7 +671,7 @@ static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipSt
         snprintf(name, sizeof name, "rfft2d_kernel<%d, %s, %d, %s>", N, WIN ? "true" : "false", NZ, RAW ? "true" : "false");
         kernel_log_add(name, blocks * FftShape<N, false, (NZ < N)>::THREADS);
     }
-    hipLaunchKernelGGL((rfft2d_kernel<N, WIN, NZ, RAW>), dim3((unsigned)blocks), dim3(FftShape<N, false, (NZ < N)>::THREADS), lds, s, j0, j1,
+    FBFC_LAUNCH((rfft2d_kernel<N, WIN, NZ, RAW>), dim3((unsigned)blocks), dim3(FftShape<N, false, (NZ < N)>::THREADS), lds, s, j0, j1,
                        j2, (unsigned)blocks0, (unsigned)blocks01);
     return hipGetLastError();
 }
@@ -743,7 +743,7 @@ static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s, const InvArgs
         snprintf(name, sizeof name, "irfft2d_kernel<%d, %s, %d>", N, WIN ? "true" : "false", PHASES);
         kernel_log_add(name, (blocks + bblocks) * S::THREADS);
     }
-    hipLaunchKernelGGL((irfft2d_kernel<N, WIN, PHASES>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
+    FBFC_LAUNCH((irfft2d_kernel<N, WIN, PHASES>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
                        j0, j1, (unsigned)blocks0, bgrad, bblocks);
     return hipGetLastError();
 }

@@ -537,7 +537,7 @@ static hipError_t launch_fwd_rows(const FwdArgs &a, const FwdArgs *second, hipSt
         snprintf(name, sizeof name, "rfft2d_rows_kernel<%d, %d, %d, %s>", N, T, NZ, RAW ? "true" : "false");
         kernel_log_add(name, blocks * S::THREADS);
     }
-    hipLaunchKernelGGL((rfft2d_rows_kernel<N, T, NZ, RAW>), dim3((unsigned)blocks), dim3(S::THREADS), lds, s, j0, j1,
+    FBFC_LAUNCH((rfft2d_rows_kernel<N, T, NZ, RAW>), dim3((unsigned)blocks), dim3(S::THREADS), lds, s, j0, j1,
                        j2, (unsigned)blocks0, (unsigned)blocks01);
     return hipGetLastError();
 }
@@ -559,7 +559,7 @@ static hipError_t launch_inv_rows(const InvArgs &a, hipStream_t s)
         snprintf(name, sizeof name, "irfft2d_rows_kernel<%d, %d>", N, T);
         kernel_log_add(name, (blocks + bblocks) * S::THREADS);
     }
-    hipLaunchKernelGGL((irfft2d_rows_kernel<N, T>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
+    FBFC_LAUNCH((irfft2d_rows_kernel<N, T>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
                        reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL, a.bias,
                        a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks);
     return hipGetLastError();

@@ -446,11 +446,11 @@ static hipError_t launch1d_tiny(bool inverse, const float *in, float *out, long 
     const long blocks = (pairs + 255) / 256;
     if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
     if (!inverse) {
-        hipLaunchKernelGGL(rfft1d_kernel<N>, dim3((unsigned)blocks), dim3(256), 0, s, in,
+        FBFC_LAUNCH(rfft1d_kernel<N>, dim3((unsigned)blocks), dim3(256), 0, s, in,
                            reinterpret_cast<float2 *>(out), rows, n, pad_l);
         kernel_log_add("rfft1d_kernel", blocks * 256);
     } else {
-        hipLaunchKernelGGL(irfft1d_kernel<N>, dim3((unsigned)blocks), dim3(256), 0, s,
+        FBFC_LAUNCH(irfft1d_kernel<N>, dim3((unsigned)blocks), dim3(256), 0, s,
                            reinterpret_cast<const float2 *>(in), out, rows, n, pad_l);
         kernel_log_add("irfft1d_kernel", blocks * 256);
     }
@@ -473,22 +473,22 @@ static hipError_t launch1d(bool inverse, const float *in, float *out, long rows,
     if (!inverse) {
         float2 *freq = reinterpret_cast<float2 *>(out);
         if (rows_vec4(in, n, pad_l))
-            hipLaunchKernelGGL((rfft1d_rows_kernel<N, 4>), grid, block, 0, s, in, freq, rows, n, pad_l);
+            FBFC_LAUNCH((rfft1d_rows_kernel<N, 4>), grid, block, 0, s, in, freq, rows, n, pad_l);
         else
-            hipLaunchKernelGGL((rfft1d_rows_kernel<N, 1>), grid, block, 0, s, in, freq, rows, n, pad_l);
+            FBFC_LAUNCH((rfft1d_rows_kernel<N, 1>), grid, block, 0, s, in, freq, rows, n, pad_l);
         kernel_log_add("rfft1d_rows_kernel", blocks * G::LANES);
     } else {
         const float2 *freq = reinterpret_cast<const float2 *>(in);
         const bool wide = (reinterpret_cast<uintptr_t>(in) & 15) == 0;  // chunks start on even complex counts
         const bool vec = rows_vec4(out, n, pad_l);
         if (vec && wide)
-            hipLaunchKernelGGL((irfft1d_rows_kernel<N, 4, 2>), grid, block, 0, s, freq, out, rows, n, pad_l);
+            FBFC_LAUNCH((irfft1d_rows_kernel<N, 4, 2>), grid, block, 0, s, freq, out, rows, n, pad_l);
         else if (vec)
-            hipLaunchKernelGGL((irfft1d_rows_kernel<N, 4, 1>), grid, block, 0, s, freq, out, rows, n, pad_l);
+            FBFC_LAUNCH((irfft1d_rows_kernel<N, 4, 1>), grid, block, 0, s, freq, out, rows, n, pad_l);
         else if (wide)
-            hipLaunchKernelGGL((irfft1d_rows_kernel<N, 1, 2>), grid, block, 0, s, freq, out, rows, n, pad_l);
+            FBFC_LAUNCH((irfft1d_rows_kernel<N, 1, 2>), grid, block, 0, s, freq, out, rows, n, pad_l);
         else
-            hipLaunchKernelGGL((irfft1d_rows_kernel<N, 1, 1>), grid, block, 0, s, freq, out, rows, n, pad_l);
+            FBFC_LAUNCH((irfft1d_rows_kernel<N, 1, 1>), grid, block, 0, s, freq, out, rows, n, pad_l);
         kernel_log_add("irfft1d_rows_kernel", blocks * G::LANES);
     }
     return hipGetLastError();
@@ -523,12 +523,13 @@ hipError_t launch_rfft2d_tiny(int N, const float *in, float *out, long planes, i
                               int pad_l, hipStream_t s)
 {
     const long blocks = (planes + 255) / 256;
-    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    if (blocks > 0x7fffffffL || (N != 2 && N != 4)) return hipErrorInvalidValue;
+    kernel_log_add(N == 2 ? "rfft2d_tiny_kernel<2>" : "rfft2d_tiny_kernel<4>", blocks * 256);
     if (N == 2)
-        hipLaunchKernelGGL(rfft2d_tiny_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s, in,
+        FBFC_LAUNCH(rfft2d_tiny_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s, in,
                            reinterpret_cast<float2 *>(out), planes, h, w, pad_u, pad_l);
     else if (N == 4)
-        hipLaunchKernelGGL(rfft2d_tiny_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, s, in,
+        FBFC_LAUNCH(rfft2d_tiny_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, s, in,
                            reinterpret_cast<float2 *>(out), planes, h, w, pad_u, pad_l);
     else
         return hipErrorInvalidValue;
@@ -539,13 +540,14 @@ hipError_t launch_irfft2d_tiny(int N, const float *in, float *out, long planes, 
                                int pad_l, const float *bias, int bias_period, hipStream_t s)
 {
     const long blocks = (planes + 255) / 256;
-    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    if (blocks > 0x7fffffffL || (N != 2 && N != 4)) return hipErrorInvalidValue;
+    kernel_log_add(N == 2 ? "irfft2d_tiny_kernel<2>" : "irfft2d_tiny_kernel<4>", blocks * 256);
     const int period = bias_period > 0 ? bias_period : 1;
     if (N == 2)
-        hipLaunchKernelGGL(irfft2d_tiny_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s,
+        FBFC_LAUNCH(irfft2d_tiny_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s,
                            reinterpret_cast<const float2 *>(in), out, planes, h, w, pad_u, pad_l, bias, period);
     else if (N == 4)
-        hipLaunchKernelGGL(irfft2d_tiny_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, s,
+        FBFC_LAUNCH(irfft2d_tiny_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, s,
                            reinterpret_cast<const float2 *>(in), out, planes, h, w, pad_u, pad_l, bias, period);
     else
         return hipErrorInvalidValue;

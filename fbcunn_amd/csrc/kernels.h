@@ -1,9 +1,25 @@
 // Internal launch interface between the C ABI (api.cpp) and the kernels.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stddef.h>
 
 namespace fbfc {
+
+// Per-launch timing.  While a pass runs with per-launch timing armed (api.cpp), every kernel launch of the
+// calling thread takes the next pair of events from the armed list and is issued with them attached to
+// the dispatch itself: their elapsed time is the kernel's own start-to-end time on the device, which is
+// what a profiler's kernel trace reports, with no event or launch overhead in it.  Unarmed (the normal
+// case) a launch is an ordinary launch.
+bool launch_events_next(hipEvent_t *start, hipEvent_t *stop);
+#define FBFC_LAUNCH(kernel, grid, block, lds, stream, ...)                                              \
+    do {                                                                                                \
+        hipEvent_t es_ = nullptr, ee_ = nullptr;                                                        \
+        if (fbfc::launch_events_next(&es_, &ee_))                                                       \
+            hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, es_, ee_, 0, __VA_ARGS__);          \
+        else                                                                                            \
+            hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                          \
+    } while (0)
 
 // fft_kernels.hip ------------------------------------------------------------
 // N in {8,16,32,64,128}; any other value returns hipErrorInvalidValue.
@@ -137,8 +153,8 @@ constexpr long kStreamBytes = 144L << 20;
 inline bool stream_bytes(long bytes) { return bytes > kStreamBytes; }
 // -1: the rule above (default); 1: non-temporal spectrum stores always (where runs are whole lines)
 void spectrum_stream_force(int v);
-// The 64x64 tile kernel with clock counters: adds every workgroup's shader-clock and 100 MHz ticks to
-// ticks[0] and ticks[1] (m, n multiples of 64, k of 16)
+// Measurement library only (built with FBFC_PROBES): the 64x64 tile kernel with clock counters, which adds
+// every workgroup's shader-clock and 100 MHz ticks to ticks[0] and ticks[1] (m, n multiples of 64, k of 16)
 hipError_t launch_cgemm_clock_probe(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
                                     int k, unsigned long long *ticks, hipStream_t s);
 

@@ -39,22 +39,27 @@ __global__ __launch_bounds__(256) void freq_to_planes_kernel(const float2 *__res
     __shared__ float2 tile[32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int q0 = blockIdx.x * 32;
-    const long p0 = (long)blockIdx.y * 32;
+    // the grid's second dimension holds at most 65535 workgroups: each walks the plane tiles with that stride
+    const long ptiles = (planes + 31) / 32;
+    for (long pt = blockIdx.y; pt < ptiles; pt += gridDim.y) {
+        const long p0 = pt * 32;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ql = ty + 8 * i;   // entry of the reference buffer handled by this row of the tile
-        if (q0 + ql < nq && p0 + tx < planes) {
-            const RefEntry e = ref_source(mode, N, q0 + ql);
-            float2 v = freq[(long)e.q * planes + p0 + tx];
-            if (e.conj) v.y = -v.y;
-            tile[ql][tx] = v;
+        for (int i = 0; i < 4; ++i) {
+            const int ql = ty + 8 * i;   // entry of the reference buffer handled by this row of the tile
+            if (q0 + ql < nq && p0 + tx < planes) {
+                const RefEntry e = ref_source(mode, N, q0 + ql);
+                float2 v = freq[(long)e.q * planes + p0 + tx];
+                if (e.conj) v.y = -v.y;
+                tile[ql][tx] = v;
+            }
         }
-    }
-    __syncthreads();
+        __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int pl = ty + 8 * i;
-        if (p0 + pl < planes && q0 + tx < nq) buf[(p0 + pl) * nq + q0 + tx] = tile[tx][pl];
+        for (int i = 0; i < 4; ++i) {
+            const int pl = ty + 8 * i;
+            if (p0 + pl < planes && q0 + tx < nq) buf[(p0 + pl) * nq + q0 + tx] = tile[tx][pl];
+        }
+        __syncthreads();  // the tile is free for the next round
     }
 }
 
@@ -68,40 +73,49 @@ __global__ __launch_bounds__(256) void planes_to_freq_kernel(const float2 *__res
     __shared__ float2 tile[32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int q0 = blockIdx.x * 32;
-    const long p0 = (long)blockIdx.y * 32;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int pl = ty + 8 * i;
-        if (p0 + pl < planes && q0 + tx < nq) tile[tx][pl] = buf[(p0 + pl) * nq + q0 + tx];
-    }
-    __syncthreads();
     const int nh = N / 2 + 1;
+    const long ptiles = (planes + 31) / 32;
+    for (long pt = blockIdx.y; pt < ptiles; pt += gridDim.y) {
+        const long p0 = pt * 32;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ql = ty + 8 * i;
-        const int qref = q0 + ql;
-        if (qref >= nq || p0 + tx >= planes) continue;
-        const float2 v = tile[ql][tx];
-        if (mode != 2) {
-            freq[(long)ref_source(mode, N, qref).q * planes + p0 + tx] = v;
-        } else {
-            const int a = qref / N, c = qref - a * N;
-            if (c <= N / 2) freq[(long)(a * nh + c) * planes + p0 + tx] = v;
-            const int a2 = N - a, c2 = (N - c) % N;
-            if (a > 0 && a2 > N / 2 && c2 <= N / 2)
-                freq[(long)(a2 * nh + c2) * planes + p0 + tx] = make_float2(v.x, -v.y);
+        for (int i = 0; i < 4; ++i) {
+            const int pl = ty + 8 * i;
+            if (p0 + pl < planes && q0 + tx < nq) tile[tx][pl] = buf[(p0 + pl) * nq + q0 + tx];
         }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int ql = ty + 8 * i;
+            const int qref = q0 + ql;
+            if (qref >= nq || p0 + tx >= planes) continue;
+            const float2 v = tile[ql][tx];
+            if (mode != 2) {
+                freq[(long)ref_source(mode, N, qref).q * planes + p0 + tx] = v;
+            } else {
+                const int a = qref / N, c = qref - a * N;
+                if (c <= N / 2) freq[(long)(a * nh + c) * planes + p0 + tx] = v;
+                const int a2 = N - a, c2 = (N - c) % N;
+                if (a > 0 && a2 > N / 2 && c2 <= N / 2)
+                    freq[(long)(a2 * nh + c2) * planes + p0 + tx] = make_float2(v.x, -v.y);
+            }
+        }
+        __syncthreads();  // the tile is free for the next round
     }
 }
 
-static bool layout_args_ok(long planes, int nq) { return planes > 0 && nq > 0 && (planes + 31) / 32 <= 65535; }
+static bool layout_args_ok(long planes, int nq) { return planes > 0 && nq > 0; }
+static unsigned plane_grid(long planes)
+{
+    const long ptiles = (planes + 31) / 32;
+    return (unsigned)(ptiles < 65535 ? ptiles : 65535);
+}
 
 hipError_t launch_freq_to_planes(const float *freq, float *buf, long planes, int nq, int N, int mode,
                                  hipStream_t s)
 {
     if (!layout_args_ok(planes, nq)) return hipErrorInvalidValue;
-    kernel_log_add("freq_to_planes_kernel", (long)((nq + 31) / 32) * ((planes + 31) / 32) * 256);
-    hipLaunchKernelGGL(freq_to_planes_kernel, dim3((nq + 31) / 32, (unsigned)((planes + 31) / 32)), dim3(256), 0, s,
+    kernel_log_add("freq_to_planes_kernel", (long)((nq + 31) / 32) * plane_grid(planes) * 256);
+    FBFC_LAUNCH(freq_to_planes_kernel, dim3((nq + 31) / 32, plane_grid(planes)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(freq), reinterpret_cast<float2 *>(buf), planes, nq, N, mode);
     return hipGetLastError();
 }
@@ -110,8 +124,8 @@ hipError_t launch_planes_to_freq(const float *buf, float *freq, long planes, int
                                  hipStream_t s)
 {
     if (!layout_args_ok(planes, nq)) return hipErrorInvalidValue;
-    kernel_log_add("planes_to_freq_kernel", (long)((nq + 31) / 32) * ((planes + 31) / 32) * 256);
-    hipLaunchKernelGGL(planes_to_freq_kernel, dim3((nq + 31) / 32, (unsigned)((planes + 31) / 32)), dim3(256), 0, s,
+    kernel_log_add("planes_to_freq_kernel", (long)((nq + 31) / 32) * plane_grid(planes) * 256);
+    FBFC_LAUNCH(planes_to_freq_kernel, dim3((nq + 31) / 32, plane_grid(planes)), dim3(256), 0, s,
                        reinterpret_cast<const float2 *>(buf), reinterpret_cast<float2 *>(freq), planes, nq, N, mode);
     return hipGetLastError();
 }

@@ -50,6 +50,17 @@ class _Plan:
             check(lib().fbfc_plan_create_tiled(ctypes.byref(desc), tile[0], tile[1], ctypes.byref(self.handle)))
         self.info = PlanInfo()
         check(lib().fbfc_plan_get_info(self.handle, ctypes.byref(self.info)))
+        self.backward_state = None   # None: not asked yet; True: prepared; False: no room (two halves)
+
+    def prepare_backward(self):
+        """The extra buffers of the one-grid-per-stage backward(), made once and outside the pass.  With no
+        room for them backward() runs as its two halves (same results); any other failure raises."""
+        if self.backward_state is None:
+            rc = lib().fbfc_plan_prepare_backward(self.handle)
+            if rc not in (_lib.OK, _lib.ERR_OUT_OF_MEMORY):
+                check(rc)
+            self.backward_state = rc == _lib.OK
+        return self.backward_state
 
     def close(self):
         if self.handle:
@@ -70,7 +81,7 @@ class SpatialConvolutionDirect:
     result the self-check compares with (:91-133).  Any stride.  accGradParameters assigns gradWeight
     and gradBias, like the FFT modules here."""
 
-    def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padW=0, padH=0, device="cuda"):
+    def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padW=0, padH=0, device="cuda", init=True):
         self.nInputPlane, self.nOutputPlane = nInputPlane, nOutputPlane
         self.kW, self.kH, self.dW, self.dH, self.padW, self.padH = kW, kH, dW, dH, padW, padH
         self.device = torch.device(device)
@@ -80,9 +91,10 @@ class SpatialConvolutionDirect:
         self.gradBias = torch.zeros(nOutputPlane, device=self.device)
         self.output = None
         self.gradInput = None
-        stdv = 1.0 / math.sqrt(kW * kH * nInputPlane)
-        self.weight.uniform_(-stdv, stdv)
-        self.bias.uniform_(-stdv, stdv)
+        if init:   # init=False: the caller hands in its own parameters; the random stream is left alone
+            stdv = 1.0 / math.sqrt(kW * kH * nInputPlane)
+            self.weight.uniform_(-stdv, stdv)
+            self.bias.uniform_(-stdv, stdv)
 
     def _desc(self, input):
         _check_tensor(input, "input", 4)
@@ -197,8 +209,11 @@ class SpatialConvolutionFFT:
     def debugVSCUDNN(self, pass_name, got, run_direct):
         """Compares `got` with what the direct path computes for the same pass (run_direct(module) ->
         tensor); ||direct - got|| / ||direct|| must not exceed self.prec."""
-        other = SpatialConvolutionDirect(self.nInputPlane, self.nOutputPlane, self.kW, self.kH, self.dW, self.dH,
-                                         self.padLeft, self.padUp, device=self.device)
+        other = getattr(self, "_direct_ref", None)
+        if other is None:   # made once per module, without drawing from the caller's random stream
+            other = SpatialConvolutionDirect(self.nInputPlane, self.nOutputPlane, self.kW, self.kH, self.dW, self.dH,
+                                             self.padLeft, self.padUp, device=self.device, init=False)
+            self._direct_ref = other
         other.weight, other.bias = self.weight, self.bias
         want = run_direct(other).double()
         norm = math.sqrt(float(torch.dot(want.flatten(), want.flatten())) + 1e-8)
@@ -331,10 +346,18 @@ class SpatialConvolutionFFT:
             raise ValueError("gradOutput has the wrong shape")
         if self.gradInput is None or self.gradInput.shape != input.shape:
             self.gradInput = torch.empty_like(input)
+        plan.prepare_backward()   # allocates on the first call for this shape only (see prepareBackward)
         check(lib().fbfc_backward(plan.handle, _ptr(input), _ptr(gradOutput), _ptr(self.weight),
                                   _ptr(self.gradInput), _ptr(self.gradWeight), _ptr(self.gradBias),
                                   ctypes.c_float(scale), _stream()))
         return self.gradInput
+
+    def prepareBackward(self, input):
+        """Allocates what backward() on inputs of this shape needs, so that backward() itself allocates
+        nothing (call it before capturing backward() into a graph).  True if the one-grid-per-stage form
+        will run, False if there was no room and backward() will run as its two passes."""
+        self._check_input(input)
+        return self._plan_for(input.size(0), input.size(2), input.size(3)).prepare_backward()
 
     def cleanupBuffers(self):
         for plan in self._plans.values():
@@ -539,25 +562,6 @@ def transposeMM(A, B, C, invNorm, conjugateTransposeA, conjugateTransposeB, accu
                                   int(bool(conjugateTransposeA)), int(bool(conjugateTransposeB)),
                                   int(bool(accumulate)), _stream()))
     return C
-
-
-def contractionClock(mode, A, B, C, launches=20):
-    """Shader clock (MHz) the 64x64 tile contraction kernel runs at over `launches` back-to-back launches
-    of C = op(A, B) (mode 0: A conj(B)^T, 1: A B, 2: conj(A)^T B; operands (Q, rows, cols, 2) as for
-    transposeMM); C receives the unscaled product.  A measurement aid: the MFMA peak is quoted at the
-    chip's peak clock, sustained fp32 MFMA work runs below it."""
-    for t, nme in ((A, "A"), (B, "B"), (C, "C")):
-        _check_tensor(t, nme, 4)
-    Q, m, n = C.size(0), C.size(1), C.size(2)
-    k = A.size(1) if mode == 2 else A.size(2)
-    exp_a = (Q, k, m, 2) if mode == 2 else (Q, m, k, 2)
-    exp_b = (Q, n, k, 2) if mode == 0 else (Q, k, n, 2)
-    if mode not in (0, 1, 2) or tuple(A.shape) != exp_a or tuple(B.shape) != exp_b:
-        raise ValueError("operand shapes do not match: A %s B %s C %s" % (tuple(A.shape), tuple(B.shape), tuple(C.shape)))
-    mhz = ctypes.c_float(0.0)
-    check(lib().fbfc_debug_contraction_clock(mode, _ptr(A), _ptr(B), _ptr(C), Q, m, n, k, int(launches),
-                                             ctypes.byref(mhz), _stream()))
-    return float(mhz.value)
 
 
 def updateOutputBias(output, bias):

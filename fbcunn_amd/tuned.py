@@ -33,6 +33,9 @@ class SpatialConvolution:
     maximalMemoryOverhead, inferenceOnly)."""
 
     reportErrors = False
+    # the direct candidate is plain, untuned code: above this many FLOPs per pass it is timed on a slice of
+    # the batch and the time scaled up, so that tuning a large layer does not spend seconds on it
+    directTimingFlops = 20e9
 
     def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padLeft=0, padUp=0,
                  maximalMemoryOverhead=None, inferenceOnly=False, device="cuda"):
@@ -85,12 +88,14 @@ class SpatialConvolution:
         except _lib.FbfcError:
             return None
         sizes = (info.input_freq_bytes, info.weight_freq_bytes, info.output_freq_bytes)
-        return sum(sizes) + (max(sizes) if reuse != nn.SpatialConvolutionFFT.memoryReuseNone else 0)
+        # + the result buffer of a reuse policy, + what backward() adds (training only)
+        return (sum(sizes) + (max(sizes) if reuse != nn.SpatialConvolutionFFT.memoryReuseNone else 0)
+                + (0 if self.inferenceOnly else info.backward_freq_bytes))
 
     def _make(self, cls, tile, reuse):
         args = (self.inputPlanes, self.outputPlanes, self.kW, self.kH, self.dW, self.dH, self.padLeft, self.padUp)
         if cls == "SpatialConvolutionDirect":
-            inst = nn.SpatialConvolutionDirect(*args, device=self.device)
+            inst = nn.SpatialConvolutionDirect(*args, device=self.device, init=False)
         elif tile is None:
             inst = getattr(nn, cls)(*args, reuse, device=self.device)
         else:
@@ -99,12 +104,9 @@ class SpatialConvolution:
         inst.gradWeight, inst.gradBias = self.gradWeight, self.gradBias
         return inst
 
-    def _tune(self, input):
+    def _pick(self, input, grad_output):
+        """Times every candidate and returns (winner, its ms); raises if none runs or the self-check fails."""
         B, _, iH, iW = input.shape
-        oH, oW = (iH + 2 * self.padUp - self.kH) // self.dH + 1, (iW + 2 * self.padLeft - self.kW) // self.dW + 1
-        grad_output = torch.zeros(B, self.outputPlanes, max(oH, 1), max(oW, 1), device=input.device)
-        # tuning must not disturb the caller's gradients
-        keep_gw, keep_gb = self.gradWeight.clone(), self.gradBias.clone()
         best, best_ms = None, float("inf")
         self.timings = {}
         for cls, tile, reuse in self._candidates(iH, iW):
@@ -117,12 +119,18 @@ class SpatialConvolution:
                 self.timings[key] = {"memoryConsumption": nbytes, "skipped": "exceeds maximalMemoryOverhead"}
                 continue
             inst = self._make(cls, tile, reuse)
+            x_t, g_t, factor = input, grad_output, 1.0
+            if cls == "SpatialConvolutionDirect":
+                flops = 2.0 * B * self.outputPlanes * self.inputPlanes * grad_output.size(2) * grad_output.size(3) * self.kH * self.kW
+                if flops > self.directTimingFlops and B > 1:
+                    nb = max(1, int(B * self.directTimingFlops / flops))
+                    x_t, g_t, factor = input[:nb], grad_output[:nb], B / float(nb)
             try:
-                t1 = _time_function(inst.updateOutput, input)
+                t1 = factor * _time_function(inst.updateOutput, x_t)
                 t2 = t3 = 0.0
                 if not self.inferenceOnly:
-                    t2 = _time_function(inst.updateGradInput, input, grad_output)
-                    t3 = _time_function(inst.accGradParameters, input, grad_output, 1.0)
+                    t2 = factor * _time_function(inst.updateGradInput, x_t, g_t)
+                    t3 = factor * _time_function(inst.accGradParameters, x_t, g_t, 1.0)
             except _lib.FbfcError as err:
                 if self.reportErrors:
                     print("%s tile %s: %s" % (cls, tile, err))
@@ -152,8 +160,19 @@ class SpatialConvolution:
             if not best.cudnnChecks:
                 best.cleanupBuffers()
                 raise _lib.FbfcError(_lib.ERR_HIP, "self-check of %s against the direct convolution failed" % (self.bestKey,))
-        self.gradWeight.copy_(keep_gw)
-        self.gradBias.copy_(keep_gb)
+        return best, best_ms
+
+    def _tune(self, input):
+        B, _, iH, iW = input.shape
+        oH, oW = (iH + 2 * self.padUp - self.kH) // self.dH + 1, (iW + 2 * self.padLeft - self.kW) // self.dW + 1
+        grad_output = torch.zeros(B, self.outputPlanes, max(oH, 1), max(oW, 1), device=input.device)
+        # tuning must not disturb the caller's gradients, whichever way it ends
+        keep_gw, keep_gb = self.gradWeight.clone(), self.gradBias.clone()
+        try:
+            best, best_ms = self._pick(input, grad_output)
+        finally:
+            self.gradWeight.copy_(keep_gw)
+            self.gradBias.copy_(keep_gb)
         if self.reportLevel >= 1:
             print("Best FFT: ", best_ms, " ", self.bestKey)
         self.bestModuleInst = best

@@ -64,6 +64,8 @@ typedef struct {
     size_t output_freq_bytes;  /* Q * B * F * 8 */
     size_t scratch_bytes;      /* what fbfc_acc_grad_parameters_bias needs for this shape */
     int tiles_h, tiles_w;      /* output tiles per image (1 x 1 for an untiled plan) */
+    size_t backward_freq_bytes; /* what fbfc_plan_prepare_backward adds: input_freq_bytes +
+                                   weight_freq_bytes for an untiled plan, 0 for a tiled one */
 } fbfc_plan_info;
 
 typedef struct fbfc_plan fbfc_plan;
@@ -139,13 +141,21 @@ int fbfc_acc_grad_parameters(fbfc_plan *plan, const float *input, const float *g
  * gradOutput the first one computed (the reference passes its outputTransposeBuffer in the
  * reuse list) whatever the plan's reuse policy.  Tiled plans recompute it (their two passes
  * window gradOutput differently).  Results equal those of the two separate calls, bit for bit.
- * For an untiled plan each stage of the two passes is issued as one grid (the forward
- * transforms of gradOutput, weight and input; both contractions; both inverse transforms with
- * the bias gradient), which needs the two product spectra in buffers of their own: the first
- * call allocates input_freq_bytes + weight_freq_bytes more device memory and keeps it until
- * the plan is destroyed.  If that allocation fails the pass runs as its two halves. */
+ * For an untiled plan on which fbfc_plan_prepare_backward has succeeded each stage of the two
+ * passes is issued as one grid (the forward transforms of gradOutput, weight and input; both
+ * contractions; both inverse transforms with the bias gradient); otherwise the pass runs as its
+ * two halves.  Like every pass it allocates nothing. */
 int fbfc_backward(fbfc_plan *plan, const float *input, const float *grad_output, const float *weight,
                   float *grad_input, float *grad_weight, float *grad_bias, float scale, void *stream);
+
+/* Gives an untiled plan the two buffers the one-grid-per-stage form of fbfc_backward writes its
+ * product spectra to (it reads all three operand spectra in one launch, so neither result may
+ * overwrite one of them): backward_freq_bytes more device memory on the plan's device, kept until the
+ * plan is destroyed.  Call it once, outside any stream capture.  FBFC_ERR_OUT_OF_MEMORY if there is
+ * no room (fbfc_backward then keeps running as its two halves); a no-op for tiled plans and for a
+ * plan that is prepared already.  No counterpart in the reference, whose modules allocate inside
+ * their passes (fbcunn/SpatialConvolutionFFT.lua:652-688). */
+int fbfc_plan_prepare_backward(fbfc_plan *plan);
 
 /* Memory-reuse policy of the module (SpatialConvolutionFFT.lua:59-63,216-240;
  * used at SpatialConvolutionFBFFT.lua:226-230,305-322): with a flag set, the
@@ -161,7 +171,11 @@ int fbfc_plan_set_reuse(fbfc_plan *plan, unsigned flags);
  * on the pass's stream (stages are pure functions of their inputs, so results are
  * unchanged) and synchronises at the end; fbfc_plan_stage_ms then reports the mean time
  * of one launch.  The launches are those of an untimed pass.  reps = 0 switches timing
- * off.  Stage slots: */
+ * off.  reps < 0: the pass runs exactly as an untimed one, every launch once, and each launch is
+ * timed by the start and end of its own dispatch on the device (what a profiler's kernel trace
+ * reports as the kernel's duration: no launch gap, no event overhead); a stage reports the sum
+ * over its launches.  This is the duration of the kernel inside an ordinary pass, with its
+ * operands wherever the previous kernel left them.  Stage slots: */
 enum { FBFC_STAGE_FFT_A = 0,   /* the forward-FFT launch: both operands of the pass, or the
                                   first one alone when the second is reused */
        FBFC_STAGE_FFT_B = 1,   /* the second operand alone (when the first is reused) */
@@ -188,17 +202,6 @@ int fbfc_debug_force_contraction_kernel(int variant);
  * non-temporal stores; 1 = always non-temporal (where the kernel writes whole 128-byte lines).  Alone a
  * transform is about as fast either way; the pass that follows is not.  Results do not depend on it. */
 int fbfc_debug_force_spectrum_streaming(int mode);
-/* Measurement (no counterpart in the reference): the shader clock the 64x64 tile contraction kernel
- * actually runs at.  Issues `launches` back-to-back launches of the per-frequency product with clock
- * counters in the kernel and returns, for the last launch, shader-clock ticks per microsecond of
- * workgroup lifetime in *mhz.  mode 0: C = A conj(B)^T with A (Q, m, k), B (Q, n, k) (updateOutput);
- * mode 1: C = A B with B (Q, k, n) (updateGradInput); mode 2: C = conj(A)^T B with A (Q, k, m),
- * B (Q, k, n) (accGradParameters); C (Q, m, n) is written unscaled.  m, n multiples of 64, k of 16,
- * 16-byte aligned operands.  The MFMA peak is quoted at the 2.4 GHz peak clock; under sustained fp32 MFMA load the chip
- * runs lower, and this is the number that says how much lower.  Synchronises the stream. */
-int fbfc_debug_contraction_clock(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
-                                 int k, int launches, float *mhz, void *stream);
-
 /* Stand-alone stages ------------------------------------------------------------
  * Replaces FFTWrapper_fft with fbfft (src/fft/FFTWrapperLua.cpp:209-272 ->
  * fbfft2dHost, src/fft/FBFFTHost.cpp:39-116): batched 2-D real-to-complex FFT of
@@ -215,7 +218,9 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
  * plane (the fused form of updateOutputBiasFFI, src/ConvolutionBias.cu:39-51).
  * As in any complex-to-real transform the input is taken to be the spectrum of a real
  * plane: the entries (ky > N/2, kx in {0, N/2}) are not read but taken as the
- * conjugates of (N - ky, kx). */
+ * conjugates of (N - ky, kx), and the imaginary parts of the four self-conjugate entries
+ * (ky in {0, N/2}, kx in {0, N/2}) are ignored (sizes 8 to 128; sizes 2 and 4 read every entry
+ * and keep the real part of the result). */
 int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l,
                 int fft_size, float *real, const float *bias, int bias_period, void *stream);
 
@@ -226,7 +231,11 @@ int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad
  * N > 32 (test/test_FFTModule.lua:238-241).  workspace: fbfc_planes_layout_workspace_bytes(planes, N)
  * bytes of device memory, the counterpart of the buffer tensor the reference passes for sizes above
  * 32 (fbcunn/FFTWrapper.lua:73-79, 114-122); the transform runs frequency-major in it and one more
- * kernel converts the layout.  The inverse is unnormalised and reads the whole half plane given. */
+ * kernel converts the layout.  The inverse is unnormalised and, like fbfc_ifft2d, takes its input
+ * to be the spectrum of a real plane: of the half plane given, the entries the frequency-major
+ * spectrum holds twice over -- (ky > N/2, kx in {0, N/2}), which repeat (N - ky, kx) as conjugates --
+ * are not used, so the result equals the reference's exactly when the buffer is Hermitian (as every
+ * spectrum or product of spectra of real planes is, up to rounding). */
 size_t fbfc_planes_layout_workspace_bytes(long planes, int fft_size);
 int fbfc_fft2d_planes(const float *real, long planes, int h, int w, int pad_u, int pad_l,
                       int fft_size, float *freq_planes, float *workspace, void *stream);
@@ -307,7 +316,9 @@ int fbfc_acc_grad_parameters_bias_strided(const float *grad_output, float *grad_
  * hipMalloc).  It has no counterpart in the reference.  The partial sums live in a fixed 256 KB
  * array in device memory that every GPU the library runs on holds until the process ends; the call
  * allocates and frees nothing.  At most 4096 planes (FBFC_ERR_UNSUPPORTED_SIZE beyond, with the
- * limit in the message).  Results equal those of fbfc_acc_grad_parameters_bias bit for bit.  All
+ * limit in the message).  Results equal those of fbfc_acc_grad_parameters_bias bit for bit.  The
+ * first call on a device looks the array's address up (a module query, not an allocation): make it
+ * outside stream capture, or create any plan on that device first, which does the same lookup.  All
  * calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
  * threads) race and must be serialised by the caller. */
 int fbfc_acc_grad_parameters_bias_noalloc(const float *grad_output, float *grad_bias, float scale,

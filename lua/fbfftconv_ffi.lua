@@ -12,7 +12,7 @@ typedef struct { int batch, in_planes, out_planes, in_h, in_w, k_h, k_w,
                  stride_h, stride_w, pad_h, pad_w; } fbfc_conv_desc;
 typedef struct { int fft_size, n_freq, out_h, out_w;
                  size_t input_freq_bytes, weight_freq_bytes, output_freq_bytes, scratch_bytes;
-                 int tiles_h, tiles_w; } fbfc_plan_info;
+                 int tiles_h, tiles_w; size_t backward_freq_bytes; } fbfc_plan_info;
 typedef struct fbfc_plan fbfc_plan;
 
 const char *fbfc_version(void);
@@ -32,6 +32,7 @@ int fbfc_acc_grad_parameters(fbfc_plan *plan, const float *input, const float *g
                              float *grad_weight, float *grad_bias, float scale, void *stream);
 int fbfc_backward(fbfc_plan *plan, const float *input, const float *grad_output, const float *weight,
                   float *grad_input, float *grad_weight, float *grad_bias, float scale, void *stream);
+int fbfc_plan_prepare_backward(fbfc_plan *plan);
 enum { FBFC_REUSE_NONE = 0, FBFC_REUSE_INPUT = 1, FBFC_REUSE_OUTPUT = 2, FBFC_REUSE_WEIGHT = 4,
        FBFC_REUSE_ALL = 7 };
 int fbfc_plan_set_reuse(fbfc_plan *plan, unsigned flags);
@@ -42,8 +43,6 @@ int fbfc_plan_stage_ms(const fbfc_plan *plan, float *ms, int n);
 int fbfc_plan_stage_kernel(const fbfc_plan *plan, int stage, char *name, size_t n);
 int fbfc_debug_force_contraction_kernel(int variant);
 int fbfc_debug_force_spectrum_streaming(int mode);
-int fbfc_debug_contraction_clock(int mode, const float *A, const float *B, float *C, int n_freq, int m, int n,
-                                 int k, int launches, float *mhz, void *stream);
 int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_l, int fft_size,
                float *freq, void *stream);
 int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l, int fft_size,

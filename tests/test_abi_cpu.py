@@ -23,6 +23,40 @@ def test_library_exports_every_declared_symbol():
     assert b"gfx950" in handle.fbfc_version()
 
 
+def test_probe_library_is_separate_from_the_shipped_one():
+    """include/fbfftconv_probe.h declares the measurement library's one symbol: libfbfftconv_probe.so
+    exports it and the shipped library does not."""
+    from fbcunn_amd import probe
+    header = open(os.path.join(ROOT, "include", "fbfftconv_probe.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(fbfc_[a-z0-9_]+)\s*\(", header))
+    assert declared == {"fbfc_probe_contraction_clock"}
+    for name in declared:
+        assert hasattr(probe.lib(), name)
+        assert not hasattr(_lib.lib(), name)
+
+
+def test_backward_buffers_are_reported():
+    info = _q(batch=128, in_planes=64, out_planes=64, in_h=27, in_w=27, k_h=5, k_w=5, pad_h=2, pad_w=2)
+    assert info.backward_freq_bytes == info.input_freq_bytes + info.weight_freq_bytes
+    assert _q(in_h=112, in_w=112, tile_h=32, tile_w=32).backward_freq_bytes == 0
+    assert _lib.lib().fbfc_plan_prepare_backward(None) == _lib.ERR_INVALID_ARGUMENT
+
+
+def test_planes_layout_entries_validate_before_launching():
+    """Every argument of the plane-major entry points is checked before the first kernel is launched
+    (no GPU needed to see the refusals)."""
+    import ctypes
+    L = _lib.lib()
+    ok, odd = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1004)
+    assert L.fbfc_ifft2d_planes(ok, 4, 9, 8, 0, 0, 8, ok, ok, None) == _lib.ERR_INVALID_ARGUMENT
+    assert b"must fit" in L.fbfc_last_error()
+    assert L.fbfc_ifft2d_planes(odd, 4, 8, 8, 0, 0, 8, ok, ok, None) == _lib.ERR_INVALID_ARGUMENT
+    assert L.fbfc_fft2d_planes(ok, 4, 8, 8, 0, 0, 8, odd, ok, None) == _lib.ERR_INVALID_ARGUMENT
+    assert L.fbfc_transpose_mm_planes(ok, odd, ok, 1, 4, 4, 4, ctypes.c_float(1.0), 0, 0, 0, ok, None) == _lib.ERR_INVALID_ARGUMENT
+    assert L.fbfc_transpose_mm_planes(ok, ok, ok, 1, 4, 4, 4, ctypes.c_float(1.0), 1, 1, 0, ok, None) == _lib.ERR_UNSUPPORTED_DIMENSION
+
+
 def _q(**kw):
     base = dict(batch=2, in_planes=3, out_planes=4, in_h=13, in_w=13, k_h=3, k_w=3,
                 stride_h=1, stride_w=1, pad_h=1, pad_w=1)

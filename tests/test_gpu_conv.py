@@ -148,6 +148,14 @@ def test_config5_large_kernel_sampled(nn, oracle):
     _close(gw[fs][:, ps], oracle.cross_correlation_reverse_valid(x[:, ps], g[:, fs], (1, 1), 1.0, p4),
            "config 5 gradWeight")
     _close(gb, oracle.bias_acc_grad_parameters(g, 1.0), "config 5 gradBias")
+    # a second slice that straddles the contraction's tile borders (64 images, filter planes 64 and 192,
+    # input planes in the last 32-wide block) and the transforms' plane groups (test/test_FFT.lua:160-256
+    # compares whole tensors; here every sampled value still sums over all contracted planes)
+    bs, fs, ps = [1, 31, 62], list(range(60, 69)) + list(range(250, 256)), list(range(90, 96))
+    _close(out[bs][:, fs], oracle.cross_correlation_valid(x[bs], w[fs], (1, 1), p4), "config 5 output, slice 2")
+    _close(gin[bs][:, ps], oracle.convolution_full(g[bs], w[:, ps], (1, 1), p4), "config 5 gradInput, slice 2")
+    _close(gw[fs][:, ps], oracle.cross_correlation_reverse_valid(x[:, ps], g[:, fs], (1, 1), 1.0, p4),
+           "config 5 gradWeight, slice 2")
     # size-independent property on the whole tensors: <out, g> = <x, gradInput> = <w, gradWeight>
     lhs = float(torch.dot(net.output.double().flatten(), gd.double().flatten()))
     assert abs(lhs - float(torch.dot(xd.double().flatten(), net.gradInput.double().flatten()))) <= 1e-4 * abs(lhs)
@@ -403,3 +411,36 @@ def test_spectrum_store_policy_does_not_change_results(nn):
     for other in results[1:]:
         for a, b in zip(results[0], other):
             assert np.isfinite(a).all() and np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("shape", [(16, 32, 32, 3, 13, 1), (2, 8, 24, 9, 55, 4)])
+def test_timed_passes_give_the_untimed_results(nn, shape):
+    """fbfc_plan_set_timed: with repetitions (reps > 0) and with per-launch dispatch timing (reps < 0) a pass
+    makes the launches of an untimed one, so every result keeps its bits; every stage that ran reports a
+    positive time, and the per-launch figure of a stage is no longer than the same stage between two events."""
+    B, P, F, k, H, pad = shape
+    o = H + 2 * pad - k + 1
+    net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad)
+    net.weight.copy_(dev(synth.normal(8, (F, P, k, k), 0.0, 0.05, stream=1)))
+    net.bias.copy_(dev(synth.uniform(8, (F,), -0.1, 0.1, stream=2)))
+    x, g = dev(synth.uniform(8, (B, P, H, H), stream=0)), dev(synth.uniform(8, (B, F, o, o), stream=3))
+
+    def step():
+        net.updateOutput(x)
+        net.updateGradInput(x, g)
+        net.accGradParameters(x, g, 0.5)
+        return [host(t).copy() for t in (net.output, net.gradInput, net.gradWeight, net.gradBias)]
+
+    want = step()
+    times = {}
+    for reps in (1, 3, -1):
+        net.timed = reps
+        got = step()
+        for a, b in zip(got, want):
+            assert np.array_equal(a, b), "timed = %d changes a result" % reps
+        times[reps] = net.stageTimes(x)               # of the last pass, accGradParameters
+        assert times[reps]["mm"] > 0 and times[reps]["ifft"] > 0 and times[reps]["fft_a"] > 0
+    net.timed = False
+    for s in ("fft_a", "mm", "ifft"):
+        assert times[-1][s] <= times[1][s] * 1.05 + 0.002, (s, times)
+    net.cleanupBuffers()

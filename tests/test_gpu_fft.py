@@ -336,3 +336,57 @@ def test_round_trip_in_the_reference_layout(nn):
     back = torch.empty_like(xd)
     w.ffti(back, freq, 2)
     assert np.abs(host(back) / (n * n) - x).max() <= 1e-5 * np.abs(x).max()
+
+
+@pytest.mark.parametrize("n,planes", [(8, 40), (16, 70), (32, 33), (64, 21), (64, 9), (128, 5)])
+def test_inverse_takes_its_input_as_the_spectrum_of_a_real_plane(nn, n, planes):
+    """What the header documents for a buffer that is not exactly Hermitian (rounding breaks the symmetry of
+    a product of spectra): the entries (ky > N/2, kx in {0, N/2}) are not read, and the imaginary parts of
+    the four self-conjugate entries do not count.  Garbage there, NaN included, leaves every output bit
+    unchanged, in the frequency-major and in the reference's plane-major layout."""
+    h = w = n - 3
+    x = synth.uniform(700 + n, (planes, n, n))
+    spec = np.fft.rfft2(x.astype(np.float64))                    # (planes, N, N/2+1): X[ky][kx]
+    clean = planes_to_freq_major(spec)
+    dirty = clean.copy()                                          # (N, N/2+1, planes, 2)
+    for kx in (0, n // 2):
+        dirty[n // 2 + 1:, kx] = np.nan
+        for ky in (0, n // 2):
+            dirty[ky, kx, :, 1] = 123.0
+    outs = []
+    for buf in (clean, dirty):
+        out = torch.full((planes, h, w), float("nan"), device="cuda")
+        nn.FFTWrapper("fbfft", 1, 2).ffti(out, dev(buf))
+        outs.append(host(out))
+    assert np.isfinite(outs[0]).all()
+    assert np.array_equal(outs[0], outs[1])
+    want = x[:, 2:2 + h, 1:1 + w].astype(np.float64) * (n * n)
+    assert np.abs(outs[0] - want).max() <= TOL * np.abs(want).max() * 4
+    # plane-major: the same entries of X, wherever the reference's half plane keeps them
+    full = np.fft.fft2(x.astype(np.float64))
+    ref_clean = _reference_layout(full, n)
+    ref_dirty = ref_clean.copy()
+    bad = np.zeros((n, n), bool)                                  # [ky][kx] entries that are not used
+    for kx in (0, n // 2):
+        bad[n // 2 + 1:, kx] = True
+    bad_ref = _reference_layout(np.broadcast_to(bad, (1, n, n)), n)[0]
+    ref_dirty[:, bad_ref] = np.nan
+    outs = []
+    for spec_ref in (ref_clean, ref_dirty):
+        buf = dev(np.stack([spec_ref.real, spec_ref.imag], -1).astype(np.float32))
+        out = torch.full((planes, h, w), float("nan"), device="cuda")
+        nn.FFTWrapper("fbfft", 1, 2, layout="planes").ffti(out, buf)
+        outs.append(host(out))
+    assert np.isfinite(outs[0]).all()
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_tiny_transforms_log_their_launch(nn):
+    w = nn.FFTWrapper("fbfft")
+    for n in (2, 4):
+        x = dev(synth.uniform(n, (300, n, n)))
+        freq = torch.empty((n, n // 2 + 1, 300, 2), device="cuda")
+        w.fft(x, freq)
+        assert w.lastKernel().startswith("rfft2d_tiny_kernel<%d> grid=" % n)
+        w.ffti(x, freq)
+        assert w.lastKernel().startswith("irfft2d_tiny_kernel<%d> grid=" % n)

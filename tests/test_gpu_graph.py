@@ -51,8 +51,8 @@ def test_passes_replay_from_a_graph(B, P, F, k, H, pad):
 
 @pytest.mark.parametrize("B,P,F,k,H,pad", [(64, 64, 128, 3, 13, 1), (4, 16, 48, 5, 27, 2)])
 def test_backward_replays_from_a_graph(B, P, F, k, H, pad):
-    """backward() with one grid per stage: its first call makes the two extra spectrum buffers, every
-    later call allocates nothing and can be captured."""
+    """backward() with one grid per stage: prepareBackward() makes the two extra spectrum buffers, the pass
+    itself allocates nothing and can be captured."""
     from fbcunn_amd import nn
     o = H + 2 * pad - k + 1
     net = nn.SpatialConvolutionFBFFT(P, F, k, k, 1, 1, pad, pad)
@@ -64,8 +64,10 @@ def test_backward_replays_from_a_graph(B, P, F, k, H, pad):
         net.backward(x, g, 0.5)
 
     results = lambda: [net.output, net.gradInput, net.gradWeight, net.gradBias]
+    assert net.prepareBackward(x) is True
     step()
     torch.cuda.synchronize()
+    assert "cgemm_backward_kernel" in net.stageKernels(x)["mm"]   # the one-grid-per-stage form ran
     want = [host(t).copy() for t in results()]
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())

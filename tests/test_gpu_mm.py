@@ -128,7 +128,7 @@ def test_transpose_mm_on_the_reference_operand_layout(nn, mode):
 
 @pytest.mark.parametrize("mode", [0, 1, 2])
 def test_contraction_clock_probe(nn, mode):
-    """The measurement variant of the tile kernel: same product as transposeMM (it runs the same tile code),
+    """The measurement variant of the tile kernel (in the probe library): same product as transposeMM (it runs the same tile code),
     and a shader clock between the chip's idle and peak clocks."""
     Q, m, n, k = 40, 128, 64, 64
     A = synth.uniform(5, (Q, k, m, 2) if mode == 2 else (Q, m, k, 2))
@@ -136,11 +136,12 @@ def test_contraction_clock_probe(nn, mode):
     C = torch.full((Q, m, n, 2), float("nan"), device="cuda")
     want = torch.empty_like(C)
     nn.transposeMM(dev(A), dev(B), want, 1.0, mode == 2, mode == 0, False)
-    mhz = nn.contractionClock(mode, dev(A), dev(B), C, launches=5)
+    from fbcunn_amd import probe
+    mhz = probe.contractionClock(mode, dev(A), dev(B), C, launches=5)
     assert 300.0 < mhz < 2600.0, mhz
     got, ref = _c(host(C)), _c(host(want))
     assert np.isfinite(got).all()
     assert np.abs(got - ref).max() <= TOL * np.abs(ref).max()
-    with pytest.raises(nn.FbfcError):
-        nn.contractionClock(mode, dev(A)[:, :, :40].contiguous() if mode != 2 else dev(A)[:, :40].contiguous(),
-                            dev(B)[:, :, :40].contiguous() if mode == 0 else dev(B)[:, :40].contiguous(), C)
+    with pytest.raises(ValueError):
+        probe.contractionClock(mode, dev(A)[:, :, :40].contiguous() if mode != 2 else dev(A)[:, :40].contiguous(),
+                               dev(B)[:, :, :40].contiguous() if mode == 0 else dev(B)[:, :40].contiguous(), C)

@@ -135,10 +135,12 @@ def test_self_check_hook(fbnn):
     for cls, extra in (("SpatialConvolutionFBFFT", ()), ("SpatialConvolutionFFTTiled", (16, 16))):
         net = getattr(nn, cls)(P, F, k, k, 1, 1, pad, pad, *extra)
         net.cudnnDebug = True
+        state = torch.cuda.get_rng_state()
         net.updateOutput(x)
         net.updateGradInput(x, g)
         net.accGradParameters(x, g, 0.5)
         assert net.cudnnChecks, cls
+        assert torch.equal(state, torch.cuda.get_rng_state())   # the hook draws nothing from the caller's random stream
         net.prec = 1e-12                      # no float32 result is that close: the hook must notice
         net.updateOutput(x)
         assert not net.cudnnChecks
@@ -156,7 +158,12 @@ def test_self_check_hook(fbnn):
         bad.selfCheck = True
         # make sure an FFT strategy wins, so that there is something to check
         bad._candidates = lambda iH, iW: [("SpatialConvolutionFBFFT", None, "none")]
+        bad.gradWeight.fill_(3.0)
+        bad.gradBias.fill_(-2.0)
         with pytest.raises(FbfcError):
             bad.updateOutput(x)
+        # a tuning run that ends in an error still leaves the caller's gradients as they were
+        assert float(bad.gradWeight.min()) == 3.0 == float(bad.gradWeight.max())
+        assert float(bad.gradBias.min()) == -2.0 == float(bad.gradBias.max())
     finally:
         nn.SpatialConvolutionFFT.prec = old

@@ -49,3 +49,33 @@ def test_no_alloc_rejects_sizes_beyond_its_array():
                                                    ctypes.c_void_p(0))
     assert rc == _lib.ERR_UNSUPPORTED_SIZE
     assert b"4096" in lib.fbfc_last_error()
+
+
+def test_no_alloc_bias_gradient_replays_from_a_graph():
+    """After one eager call on the device (which looks the fixed array up) the entry point can be captured
+    into a graph; every replay, with eager work and a synchronisation in between, gives the eager bits."""
+    lib = _lib.lib()
+    g = dev(synth.uniform(94, (16, 40, 7, 9)))
+    B, F, h, w = g.shape
+    out = torch.full((F,), float("nan"), device="cuda")
+
+    def call():
+        _lib.check(lib.fbfc_acc_grad_parameters_bias_noalloc(g.data_ptr(), out.data_ptr(), ctypes.c_float(0.75), B, F, h, w,
+                                                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    call()
+    torch.cuda.synchronize()
+    want = host(out).copy()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(3):
+        out.fill_(float("nan"))
+        (g * 2).sum().item()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(out), want), "replay %d differs from the eager result" % rep
