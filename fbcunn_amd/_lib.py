@@ -51,6 +51,7 @@ SIGNATURES = {
     "fbfc_plan_create": (_i, [ctypes.POINTER(ConvDesc), ctypes.POINTER(_vp)]),
     "fbfc_plan_query_tiled": (_i, [ctypes.POINTER(ConvDesc), _i, _i, ctypes.POINTER(PlanInfo)]),
     "fbfc_plan_create_tiled": (_i, [ctypes.POINTER(ConvDesc), _i, _i, ctypes.POINTER(_vp)]),
+    "fbfc_plan_create_tiled_iterated": (_i, [ctypes.POINTER(ConvDesc), _i, _i, ctypes.POINTER(_vp)]),
     "fbfc_plan_destroy": (_i, [_vp]),
     "fbfc_plan_get_info": (_i, [_vp, ctypes.POINTER(PlanInfo)]),
     "fbfc_update_output": (_i, [_vp, _vp, _vp, _vp, _vp, _vp]),

@@ -18,7 +18,7 @@ PROBE_LIB = os.path.join(HERE, "libfbfftconv_probe.so")
 # (source, object name, extra flags) of the measurement library
 PROBE_SOURCES = [("cgemm_kernels.hip", "cgemm_kernels_probe.o", ["-DFBFC_PROBES"]),
                  ("probe_clock.cpp", "probe_clock.o", ["-DFBFC_PROBES"])]
-SOURCES = ["api.cpp", "fft_kernels.hip", "fft_large.hip", "fft_small.hip", "cgemm_kernels.hip", "bias_kernels.hip", "bias_noalloc.hip", "layout_kernels.hip", "direct_kernels.hip"]
+SOURCES = ["api.cpp", "fft_kernels.hip", "fft_large.hip", "fft_small.hip", "cgemm_kernels.hip", "bias_kernels.hip", "bias_noalloc.hip", "layout_kernels.hip", "direct_kernels.hip", "fused_kernels.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
@@ -36,7 +36,7 @@ FLAGS = [
 # instantiations of one kernel, and the staging variants of a transform must give the same bits.
 NO_CONTRACT = ["-ffp-contract=off"]
 EXTRA_FLAGS = {"fft_large.hip": ["-mllvm", "-simplifycfg-sink-common=false"] + NO_CONTRACT,
-               "fft_kernels.hip": NO_CONTRACT, "fft_small.hip": NO_CONTRACT}
+               "fft_kernels.hip": NO_CONTRACT, "fft_small.hip": NO_CONTRACT, "fused_kernels.hip": NO_CONTRACT}
 
 
 def _compile(src, report, obj=None, extra=()):

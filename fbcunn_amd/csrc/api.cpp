@@ -218,6 +218,9 @@ struct fbfc_plan {
     fbfc_conv_desc d;
     fbfc_plan_info info;
     bool tiled;
+    bool iterated;   // tiled, passes run as fused kernels: no feature-map spectra, only w_freq, part and scratch
+    float *part;     // iterated: partial gradWeight results, acc_ranges x F x P x kh x kw floats
+    int acc_ranges;
     pass_geom fprop, bprop, accgrad;
     int device;
     float *in_freq, *w_freq, *out_freq, *res_freq, *scratch;
@@ -405,7 +408,7 @@ int fbfc_plan_query_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fb
     return plan_query_tiled(desc, tile_h, tile_w, info);
 }
 
-static int plan_create(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **out)
+static int plan_create(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **out, bool iterated = false)
 {
     if (out == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null argument");
     *out = nullptr;
@@ -413,19 +416,37 @@ static int plan_create(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_
     const bool tiled = tile_h > 0 || tile_w > 0;
     const int rc = tiled ? fbfc_plan_query_tiled(desc, tile_h, tile_w, &info) : plan_query(desc, &info);
     if (rc != FBFC_OK) return rc;
+    size_t part_bytes = 0;
+    int acc_ranges = 0;
+    if (iterated) {
+        // the fused passes keep the spectra of the feature maps on chip: the plan owns the weight spectrum,
+        // the partial gradWeight results of accGradParameters and the bias gradient's workspace
+        const int nt_out = info.tiles_h * info.tiles_w;
+        acc_ranges = fbfc::fused_accgrad_ranges(info.fft_size, desc->batch * nt_out, desc->out_planes, desc->in_planes);
+        part_bytes = (size_t)acc_ranges * desc->out_planes * desc->in_planes * desc->k_h * desc->k_w * sizeof(float);
+        info.input_freq_bytes = 0;
+        info.output_freq_bytes = 0;
+        info.scratch_bytes += part_bytes;
+    }
     fbfc_plan *p = new (std::nothrow) fbfc_plan();
     if (p == nullptr) return fail(FBFC_ERR_OUT_OF_MEMORY, "host allocation failed");
     std::memset(p, 0, sizeof *p);
     p->d = *desc;
     p->info = info;
     p->tiled = tiled;
+    p->iterated = iterated;
+    p->acc_ranges = acc_ranges;
     set_geometry(p, tile_h, tile_w);
     hipError_t e = hipGetDevice(&p->device);
     if (e == hipSuccess) e = fbfc::fft_prepare_device();
     if (e == hipSuccess) e = fbfc::bias_grad_noalloc_prepare();
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->in_freq), info.input_freq_bytes);
+    if (e == hipSuccess && iterated) e = fbfc::fused_prepare_device();
+    if (e == hipSuccess && !iterated) e = hipMalloc(reinterpret_cast<void **>(&p->in_freq), info.input_freq_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->w_freq), info.weight_freq_bytes);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&p->out_freq), info.output_freq_bytes);
+    if (e == hipSuccess && !iterated) e = hipMalloc(reinterpret_cast<void **>(&p->out_freq), info.output_freq_bytes);
+    if (e == hipSuccess && iterated) e = hipMalloc(reinterpret_cast<void **>(&p->part), part_bytes);
+    if (e == hipSuccess && iterated)
+        e = hipMalloc(reinterpret_cast<void **>(&p->scratch), fbfc::bias_grad_scratch_bytes(desc->batch, desc->out_planes));
     if (e != hipSuccess) {
         const bool oom = (e == hipErrorOutOfMemory);
         (void)hipGetLastError();
@@ -446,9 +467,16 @@ int fbfc_plan_create_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, f
     return plan_create(desc, tile_h, tile_w, out);
 }
 
+int fbfc_plan_create_tiled_iterated(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **out)
+{
+    if (tile_h < 1 || tile_w < 1) return fail(FBFC_ERR_INVALID_ARGUMENT, "both tile sizes must be specified");
+    return plan_create(desc, tile_h, tile_w, out, true);
+}
+
 int fbfc_plan_destroy(fbfc_plan *p)
 {
     if (p == nullptr) return FBFC_OK;
+    if (p->part) (void)hipFree(p->part);
     if (p->in_freq) (void)hipFree(p->in_freq);
     if (p->w_freq) (void)hipFree(p->w_freq);
     if (p->out_freq) (void)hipFree(p->out_freq);
@@ -475,6 +503,9 @@ int fbfc_plan_set_reuse(fbfc_plan *p, unsigned flags)
 {
     if (p == nullptr) return fail(FBFC_ERR_INVALID_ARGUMENT, "null plan");
     if (flags & ~(unsigned)FBFC_REUSE_ALL) return fail(FBFC_ERR_INVALID_ARGUMENT, "unknown memory reuse policy");
+    // the fused passes keep no spectrum that could be reused: like the reference's module
+    // (SpatialConvolutionFFTTiledIterated.lua:47-48) they override any policy with "none"
+    if (p->iterated) return FBFC_OK;
     if (flags != 0 && p->res_freq == nullptr) {
         // With reuse, a pass must not overwrite a spectrum a later pass wants: its
         // result goes to a buffer of its own (the reference keys such buffers by
@@ -556,6 +587,23 @@ int fbfc_update_output(fbfc_plan *p, const float *input, const float *weight, co
     const int QH = fbfc::hermitian_count(N);
     const fbfc::FreqMap fm = fbfc::hermitian_map(N);
     StageTimer tm(p, s);
+    if (p->iterated) {
+        // weight spectrum, then one kernel: windows of the input -> spectra -> sum over input planes of
+        // I conj(W) -> inverse transform, bias, output tiles
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, weight_args(p, weight), s), "rfft2d(weight)");
+        tm.done(FBFC_STAGE_FFT_A);
+        fbfc::FusedConvArgs fa = {};
+        fa.small = input; fa.big = output; fa.w_freq = p->w_freq; fa.bias = bias;
+        fa.small_win = g.a_win; fa.big_win = g.r_win;
+        fa.small_h = g.a_h; fa.small_w = g.a_w;
+        fa.big_h = g.r_h; fa.big_w = g.r_w; fa.big_pad_u = g.r_pad_u; fa.big_pad_l = g.r_pad_l;
+        fa.n_small = d.in_planes; fa.n_big = d.out_planes; fa.w_stride_small = 1; fa.w_stride_big = d.in_planes;
+        fa.out_planes = d.out_planes; fa.in_planes = d.in_planes;
+        fa.vbatch = g.vbatch; fa.conj_w = 1; fa.alpha = 1.0f / ((float)N * (float)N);
+        FBFC_STAGE(tm, fbfc::launch_fused_conv(N, fa, s), "fused updateOutput");
+        tm.done(FBFC_STAGE_MM);
+        return tm.finish();
+    }
     const fbfc::FwdArgs fin = {input, p->in_freq, (long)g.vbatch * d.in_planes, g.a_h, g.a_w, g.a_pad_u,
                                g.a_pad_l, g.a_win, 1};
     const fbfc::FwdArgs fw = weight_args(p, weight);
@@ -593,6 +641,21 @@ int fbfc_update_grad_input(fbfc_plan *p, const float *grad_output, const float *
     const int QH = fbfc::hermitian_count(N);
     const fbfc::FreqMap fm = fbfc::hermitian_map(N);
     StageTimer tm(p, s);
+    if (p->iterated) {
+        FBFC_STAGE(tm, fbfc::launch_rfft2d_one(N, weight_args(p, weight), s), "rfft2d(weight)");
+        tm.done(FBFC_STAGE_FFT_A);
+        fbfc::FusedConvArgs fa = {};
+        fa.small = grad_output; fa.big = grad_input; fa.w_freq = p->w_freq; fa.bias = nullptr;
+        fa.small_win = g.a_win; fa.big_win = g.r_win;
+        fa.small_h = g.a_h; fa.small_w = g.a_w;
+        fa.big_h = g.r_h; fa.big_w = g.r_w; fa.big_pad_u = g.r_pad_u; fa.big_pad_l = g.r_pad_l;
+        fa.n_small = d.out_planes; fa.n_big = d.in_planes; fa.w_stride_small = d.in_planes; fa.w_stride_big = 1;
+        fa.out_planes = d.out_planes; fa.in_planes = d.in_planes;
+        fa.vbatch = g.vbatch; fa.conj_w = 0; fa.alpha = 1.0f / ((float)N * (float)N);
+        FBFC_STAGE(tm, fbfc::launch_fused_conv(N, fa, s), "fused updateGradInput");
+        tm.done(FBFC_STAGE_MM);
+        return tm.finish();
+    }
     const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)g.vbatch * d.out_planes, g.a_h, g.a_w,
                                g.a_pad_u, g.a_pad_l, g.a_win, 1};
     const fbfc::FwdArgs fw = weight_args(p, weight);
@@ -635,6 +698,23 @@ static int acc_grad_parameters(fbfc_plan *p, const float *input, const float *gr
     const int QH = fbfc::hermitian_count(N);
     const fbfc::FreqMap fm = fbfc::hermitian_map(N);
     StageTimer tm(p, s);
+    if (p->iterated) {
+        fbfc::FusedAccArgs fa = {};
+        fa.input = input; fa.grad_output = grad_output; fa.grad_weight = grad_weight; fa.part = p->part;
+        fa.in_win = g.a_win; fa.go_win = g.g_win;
+        fa.in_h = g.a_h; fa.in_w = g.a_w; fa.go_h = g.g_h; fa.go_w = g.g_w; fa.kh = d.k_h; fa.kw = d.k_w;
+        fa.out_planes = d.out_planes; fa.in_planes = d.in_planes; fa.vbatch = g.vbatch; fa.nranges = p->acc_ranges;
+        fa.alpha = scale / ((float)N * (float)N);
+        FBFC_STAGE(tm, fbfc::launch_fused_accgrad(N, fa, s), "fused accGradParameters");
+        tm.done(FBFC_STAGE_MM);
+        if (grad_bias != nullptr) {
+            // no spectrum of gradOutput exists to read the plane sums from: the stand-alone reduction
+            FBFC_STAGE(tm, fbfc::launch_bias_grad(grad_output, grad_bias, scale, d.batch, d.out_planes,
+                                                  p->info.out_h * p->info.out_w, p->scratch, s), "bias grad");
+            tm.done(FBFC_STAGE_BIAS_GRAD);
+        }
+        return tm.finish();
+    }
     const fbfc::FwdArgs fgo = {grad_output, p->out_freq, (long)g.vbatch * d.out_planes, g.g_h, g.g_w, 0, 0,
                                g.g_win, 1};
     const fbfc::FwdArgs fin = {input, p->in_freq, (long)g.vbatch * d.in_planes, g.a_h, g.a_w, g.a_pad_u,

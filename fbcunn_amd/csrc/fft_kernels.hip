@@ -29,6 +29,7 @@
 #include "bias_dc.h"
 #include "fft_regs.h"
 #include "fft_stage.h"
+#include "fft_windows.h"
 #include "kernels.h"
 #include "store_nt.h"
 
@@ -122,55 +123,6 @@ __device__ __forceinline__ void build_window_table(int4 *tbl, const Window &win,
         const long off = (b * win.d1 + c) * ((long)win.img_h * win.img_w);
         tbl[tid] = make_int4((int)(unsigned)(off & 0xffffffffL), (int)(off >> 32),
                              ty * win.step_y + win.off_y, tx * win.step_x + win.off_x);
-    }
-}
-
-// Moves the windows of planes [first, first + nph) of the workgroup between global memory and their
-// nph * h canvas rows.  Each wave takes every fourth plane, so the window corner and the plane's base
-// address are wave-uniform; its lanes sweep the window 64 elements (N <= 32: at least two rows) at a
-// time with all loads of a plane in flight together.
-template <int N, bool TO_LDS>
-__device__ __forceinline__ void copy_windows(float *smem, float *g, const int4 *tbl, int first, int nph,
-                                             int h, int w, int padL, const Window &win, int tid)
-{
-    constexpr int LDR = Canvas<N>::LDR;
-    constexpr int ITER = (N * N) / 64;
-    const int wave = tid >> 6, lane = tid & 63;
-    const int c = lane % N, r0 = lane / N;
-    for (int tl = wave; tl < nph; tl += 4) {
-        const int4 q = tbl[first + tl];
-        const int off_lo = __builtin_amdgcn_readfirstlane(q.x), off_hi = __builtin_amdgcn_readfirstlane(q.y);
-        const int y0 = __builtin_amdgcn_readfirstlane(q.z), x0 = __builtin_amdgcn_readfirstlane(q.w);
-        float *gp = g + ((((long)off_hi) << 32) | (long)(unsigned)off_lo) + x0 + c;
-        float *sp = smem + (tl * h) * LDR + padL + c;
-        const bool xok = (c < w) && ((unsigned)(x0 + c) < (unsigned)win.img_w);
-        float v[ITER];
-        if (TO_LDS) {
-#pragma unroll
-            for (int i = 0; i < ITER; ++i) {
-                const int r = r0 + i * (64 / N);
-                const int y = y0 + r;
-                const bool ok = xok && (r < h) && ((unsigned)y < (unsigned)win.img_h);
-                v[i] = ok ? gp[(long)y * win.img_w] : 0.0f;
-            }
-#pragma unroll
-            for (int i = 0; i < ITER; ++i) {
-                const int r = r0 + i * (64 / N);
-                if (r < h) sp[r * LDR] = v[i];
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < ITER; ++i) {
-                const int r = r0 + i * (64 / N);
-                v[i] = (r < h) ? sp[r * LDR] : 0.0f;
-            }
-#pragma unroll
-            for (int i = 0; i < ITER; ++i) {
-                const int r = r0 + i * (64 / N);
-                const int y = y0 + r;
-                if (xok && (r < h) && ((unsigned)y < (unsigned)win.img_h)) gp[(long)y * win.img_w] = v[i];
-            }
-        }
     }
 }
 

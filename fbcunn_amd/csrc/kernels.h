@@ -91,6 +91,40 @@ hipError_t launch_rfft2d_large(int N, const FwdArgs &a, const FwdArgs *b, hipStr
 hipError_t launch_irfft2d_large(int N, const InvArgs &a, hipStream_t s);
 hipError_t fft_large_prepare_device();
 
+// fused_kernels.hip: the fused tiled convolution (tile FFT sizes 8, 16, 32) ---------------------------
+// updateOutput / updateGradInput: result(vbatch tiles x n_big planes) = inverse transform of
+// alpha * sum over the n_small contracted planes of FFT(window) x (conj) W, W = w_freq[q][f * P + p] with
+// plane index small * w_stride_small + big * w_stride_big.
+struct FusedConvArgs {
+    const float *small;   // tensor of the contracted side (input resp. gradOutput)
+    float *big;           // result tensor (output resp. gradInput)
+    const float *w_freq;  // weight spectrum, frequency-major
+    const float *bias;    // added per big plane; nullptr: none
+    Window small_win, big_win;
+    int small_h, small_w;                       // windows of the contracted side
+    int big_h, big_w, big_pad_u, big_pad_l;     // result tiles and where they sit in the circular result
+    int n_small, n_big, w_stride_small, w_stride_big, out_planes, in_planes;
+    int vbatch;           // batch * tiles
+    int conj_w;           // 1: multiply by conj(W) (updateOutput)
+    float alpha;
+};
+hipError_t launch_fused_conv(int N, const FusedConvArgs &a, hipStream_t s);
+// accGradParameters: grad_weight(F, P, kh, kw) = alpha * sum over tiles of the k x k crop of
+// IFFT(conj(FFT(gradOutput tile)) FFT(input window)); `part` holds nranges partial results of
+// out_planes * in_planes * kh * kw floats (nranges from fused_accgrad_ranges).
+struct FusedAccArgs {
+    const float *input, *grad_output;
+    float *grad_weight, *part;
+    Window in_win, go_win;
+    int in_h, in_w, go_h, go_w, kh, kw;
+    int out_planes, in_planes, vbatch, nranges;
+    float alpha;
+};
+int fused_accgrad_ranges(int N, int vbatch, int out_planes, int in_planes);
+hipError_t launch_fused_accgrad(int N, const FusedAccArgs &a, hipStream_t s);
+// raises the dynamic-LDS limit of the fused kernels on the current device (plan creation calls it)
+hipError_t fused_prepare_device();
+
 // fft_small.hip ------------------------------------------------------------------
 // 1-D batched transforms, N in {2,4,...,128}: rows of n reals at pad_l of the N-point canvas
 // <-> (rows, N/2+1) complex, row-major; the inverse is unnormalised.

@@ -42,10 +42,12 @@ def _check_tensor(t, name, ndim=None, strided=False):
 class _Plan:
     """RAII holder of one fbfc_plan."""
 
-    def __init__(self, desc, tile=None):
+    def __init__(self, desc, tile=None, iterated=False):
         self.handle = ctypes.c_void_p(0)
         if tile is None:
             check(lib().fbfc_plan_create(ctypes.byref(desc), ctypes.byref(self.handle)))
+        elif iterated:
+            check(lib().fbfc_plan_create_tiled_iterated(ctypes.byref(desc), tile[0], tile[1], ctypes.byref(self.handle)))
         else:
             check(lib().fbfc_plan_create_tiled(ctypes.byref(desc), tile[0], tile[1], ctypes.byref(self.handle)))
         self.info = PlanInfo()
@@ -250,7 +252,7 @@ class SpatialConvolutionFFT:
         if plan is None:
             desc = ConvDesc(batch, self.nInputPlane, self.nOutputPlane, in_h, in_w, self.kH, self.kW,
                             self.dH, self.dW, self.padUp, self.padLeft)
-            plan = _Plan(desc, self._tile())
+            plan = _Plan(desc, self._tile(), self._iterated())
             if self._reuse_bits:
                 check(lib().fbfc_plan_set_reuse(plan.handle, self._reuse_bits))
             self._plans[key] = plan
@@ -260,6 +262,10 @@ class SpatialConvolutionFFT:
     def _tile(self):
         """(tileSizeH, tileSizeW) of a tiled module, None otherwise."""
         return None
+
+    def _iterated(self):
+        """Whether the passes run as the fused kernels of nn.SpatialConvolutionFFTTiledIterated."""
+        return False
 
     def _check_input(self, input):
         _check_tensor(input, "input", 4)
@@ -408,7 +414,18 @@ class SpatialConvolutionFFTTiledAsync(SpatialConvolutionFFTTiled):
 
 
 class SpatialConvolutionFFTTiledIterated(SpatialConvolutionFFTTiled):
-    """nn.SpatialConvolutionFFTTiledIterated (fbcunn/SpatialConvolutionFFTTiledIterated.lua)."""
+    """nn.SpatialConvolutionFFTTiledIterated (fbcunn/SpatialConvolutionFFTTiledIterated.lua): every pass is
+    one fused kernel per tile block (window transforms, product over the contracted planes, inverse
+    transform) that never writes a spectrum of a feature map to memory.  Like the reference's module
+    (:47-48) it overrides any memory reuse policy with "none"."""
+
+    def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padLeft=0, padUp=0,
+                 tileSizeW=None, tileSizeH=None, memoryReusePolicy=None, numCudaStreams=None, device="cuda"):
+        super().__init__(nInputPlane, nOutputPlane, kW, kH, dW, dH, padLeft, padUp, tileSizeW, tileSizeH,
+                         None, numCudaStreams, device)
+
+    def _iterated(self):
+        return True
 
 
 class FFTWrapper:

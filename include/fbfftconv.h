@@ -115,6 +115,20 @@ int fbfc_plan_get_info(const fbfc_plan *plan, fbfc_plan_info *info);
 int fbfc_plan_query_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan_info *info);
 int fbfc_plan_create_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **plan);
 
+/* nn.SpatialConvolutionFFTTiledIterated (fbcunn/SpatialConvolutionFFTTiledIterated.lua:79-123,
+ * 129-175, 180-229 -> convolveIteratedFFI, src/fft/FFTIteratedConvolution.cu:71-95): a tiled plan whose
+ * passes each run as ONE fused kernel (window transforms, product over the contracted planes, inverse
+ * transform) after the small transform of the weights, so that no spectrum of a feature map is written
+ * to memory.  Same tiling rules, errors and results as fbfc_plan_create_tiled (rounding differs in the
+ * last bits: the sums over planes run in another order); the same three pass entry points.  The plan
+ * owns the weight spectrum only: fbfc_plan_get_info reports input_freq_bytes = output_freq_bytes = 0
+ * and, in scratch_bytes, the partial-result buffer of accGradParameters.  The sum over the contracted
+ * planes is vector arithmetic, not a matrix-core contraction: the kernel is meant for layers in which
+ * one side has few planes (first and last layers), where the spectra dominate the traffic of the
+ * three-kernel pass.  Like the reference's module it takes no reuse policy (fbfc_plan_set_reuse is
+ * accepted and has no effect).  fbfc_backward runs its two passes one after the other. */
+int fbfc_plan_create_tiled_iterated(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **plan);
+
 /* Replaces SpatialConvolutionFBFFT:updateOutputFFTImpl
  * (fbcunn/SpatialConvolutionFBFFT.lua:102-183):
  * output(B,F,oH,oW) = valid cross-correlation of zero-padded input(B,P,H,W) with
@@ -218,9 +232,10 @@ int fbfc_fft2d(const float *real, long planes, int h, int w, int pad_u, int pad_
  * plane (the fused form of updateOutputBiasFFI, src/ConvolutionBias.cu:39-51).
  * As in any complex-to-real transform the input is taken to be the spectrum of a real
  * plane: the entries (ky > N/2, kx in {0, N/2}) are not read but taken as the
- * conjugates of (N - ky, kx), and the imaginary parts of the four self-conjugate entries
- * (ky in {0, N/2}, kx in {0, N/2}) are ignored (sizes 8 to 128; sizes 2 and 4 read every entry
- * and keep the real part of the result). */
+ * conjugates of (N - ky, kx) (sizes 8 to 128; sizes 2 and 4 read every entry).  Every entry that
+ * is read is used as given: where the buffer deviates from the spectrum of a real plane (say by
+ * imaginary parts in the four self-conjugate entries, ky and kx in {0, N/2}) the deviation passes
+ * linearly into the result, it is not filtered out. */
 int fbfc_ifft2d(const float *freq, long planes, int h, int w, int pad_u, int pad_l,
                 int fft_size, float *real, const float *bias, int bias_period, void *stream);
 

@@ -24,6 +24,7 @@ int fbfc_plan_destroy(fbfc_plan *plan);
 int fbfc_plan_get_info(const fbfc_plan *plan, fbfc_plan_info *info);
 int fbfc_plan_query_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan_info *info);
 int fbfc_plan_create_tiled(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **plan);
+int fbfc_plan_create_tiled_iterated(const fbfc_conv_desc *desc, int tile_h, int tile_w, fbfc_plan **plan);
 int fbfc_update_output(fbfc_plan *plan, const float *input, const float *weight, const float *bias,
                        float *output, void *stream);
 int fbfc_update_grad_input(fbfc_plan *plan, const float *grad_output, const float *weight,
@@ -120,7 +121,9 @@ function M.plan(module, input, tileH, tileW)
                                           input:size(3), input:size(4), module.kH, module.kW,
                                           module.dH, module.dW, module.padUp, module.padLeft})
       local p = ffi.new('fbfc_plan*[1]')
-      if tileH and tileW then
+      if tileH and tileW and module.fbfcIterated then
+         M.check(M.C.fbfc_plan_create_tiled_iterated(d, tileH, tileW, p))
+      elseif tileH and tileW then
          M.check(M.C.fbfc_plan_create_tiled(d, tileH, tileW, p))
       else
          M.check(M.C.fbfc_plan_create(d, p))

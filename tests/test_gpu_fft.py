@@ -341,9 +341,10 @@ def test_round_trip_in_the_reference_layout(nn):
 @pytest.mark.parametrize("n,planes", [(8, 40), (16, 70), (32, 33), (64, 21), (64, 9), (128, 5)])
 def test_inverse_takes_its_input_as_the_spectrum_of_a_real_plane(nn, n, planes):
     """What the header documents for a buffer that is not exactly Hermitian (rounding breaks the symmetry of
-    a product of spectra): the entries (ky > N/2, kx in {0, N/2}) are not read, and the imaginary parts of
-    the four self-conjugate entries do not count.  Garbage there, NaN included, leaves every output bit
-    unchanged, in the frequency-major and in the reference's plane-major layout."""
+    a product of spectra): the entries (ky > N/2, kx in {0, N/2}) are not read -- garbage there, NaN included,
+    leaves every output bit unchanged, in the frequency-major and in the reference's plane-major layout --
+    and every other entry is used as given: an imaginary part eps in the four self-conjugate entries moves
+    the result by at most 4 eps (the transform is linear and unnormalised), it is not filtered out."""
     h = w = n - 3
     x = synth.uniform(700 + n, (planes, n, n))
     spec = np.fft.rfft2(x.astype(np.float64))                    # (planes, N, N/2+1): X[ky][kx]
@@ -351,10 +352,13 @@ def test_inverse_takes_its_input_as_the_spectrum_of_a_real_plane(nn, n, planes):
     dirty = clean.copy()                                          # (N, N/2+1, planes, 2)
     for kx in (0, n // 2):
         dirty[n // 2 + 1:, kx] = np.nan
+    eps = 1e-2
+    tilted = clean.copy()
+    for kx in (0, n // 2):
         for ky in (0, n // 2):
-            dirty[ky, kx, :, 1] = 123.0
+            tilted[ky, kx, :, 1] = eps
     outs = []
-    for buf in (clean, dirty):
+    for buf in (clean, dirty, tilted):
         out = torch.full((planes, h, w), float("nan"), device="cuda")
         nn.FFTWrapper("fbfft", 1, 2).ffti(out, dev(buf))
         outs.append(host(out))
@@ -362,6 +366,8 @@ def test_inverse_takes_its_input_as_the_spectrum_of_a_real_plane(nn, n, planes):
     assert np.array_equal(outs[0], outs[1])
     want = x[:, 2:2 + h, 1:1 + w].astype(np.float64) * (n * n)
     assert np.abs(outs[0] - want).max() <= TOL * np.abs(want).max() * 4
+    assert np.isfinite(outs[2]).all()
+    assert np.abs(outs[2] - outs[0]).max() <= 4 * eps * 1.01 + TOL * np.abs(want).max()
     # plane-major: the same entries of X, wherever the reference's half plane keeps them
     full = np.fft.fft2(x.astype(np.float64))
     ref_clean = _reference_layout(full, n)

@@ -146,3 +146,72 @@ def test_tiled_errors(nn):
     with pytest.raises(FbfcError) as e:
         nn.SpatialConvolutionFFTTiled(1, 1, 3, 3, 1, 1, 0, 0, 64, 64).updateOutput(big)
     assert e.value.code == ERR_UNSUPPORTED_SIZE
+
+
+# ---- nn.SpatialConvolutionFFTTiledIterated: the fused kernels ------------------------------------------
+# batch, inputPlanes, outputPlanes, kH, kW, iH, iW, padH, padW, tileH, tileW
+ITERATED = TILED + [
+    (2, 3, 64, 3, 3, 28, 28, 1, 1, 16, 16),     # first-layer shape: weights in registers, two blocks of output planes
+    (2, 64, 3, 3, 3, 28, 28, 1, 1, 16, 16),     # last-layer shape: the contracted side in chunks
+    (1, 40, 70, 3, 3, 20, 20, 1, 1, 16, 16),    # both sides beyond one batch of planes, ragged last block
+    (2, 1, 5, 5, 5, 40, 40, 2, 2, 32, 32),      # one input plane
+    (2, 3, 70, 3, 3, 18, 18, 1, 1, 8, 8),       # tiles of 8
+    (1, 7, 33, 3, 3, 12, 12, 1, 1, 8, 8),
+]
+
+
+@pytest.mark.parametrize("problem", ITERATED)
+def test_iterated_three_passes_vs_oracle(nn, oracle, problem):
+    """Every pass as one fused kernel (plus the transform of the weights): same bars as the other modules."""
+    B, P, F, kH, kW, iH, iW, padH, padW, tH, tW = problem
+    seed = 1900 + sum(problem)
+    x, w, bias, g = _tensors(B, P, F, kH, kW, iH, iW, padH, padW, seed)
+    net = nn.SpatialConvolutionFFTTiledIterated(P, F, kW, kH, 1, 1, padW, padH, tW, tH)
+    assert net.memoryReusePolicy == ["none"]
+    net.weight.copy_(dev(w))
+    net.bias.copy_(dev(bias))
+    net.gradWeight.fill_(float("nan"))
+    net.gradBias.fill_(float("nan"))
+    xd, gd = dev(x), dev(g)
+    out = host(net.updateOutput(xd))
+    kernels = net.stageKernels(xd)
+    assert "fused_conv_kernel" in kernels["mm"] and "ifft" not in kernels, kernels
+    gin = host(net.updateGradInput(xd, gd))
+    assert "fused_conv_kernel" in net.stageKernels(xd)["mm"]
+    net.accGradParameters(xd, gd, 0.41)
+    assert "fused_accgrad_kernel" in net.stageKernels(xd)["mm"]
+    gw, gb = host(net.gradWeight), host(net.gradBias)
+    net.cleanupBuffers()
+    pad = (padH, padH, padW, padW)
+    _close(out, oracle.bias_update_output(oracle.cross_correlation_valid(x, w, (1, 1), pad), bias), "output")
+    _close(gin, oracle.convolution_full(g, w, (1, 1), pad), "gradInput")
+    _close(gw, oracle.cross_correlation_reverse_valid(x, g, (1, 1), 0.41, pad), "gradWeight")
+    _close(gb, oracle.bias_acc_grad_parameters(g, 0.41), "gradBias")
+
+
+def test_iterated_first_layer_112(nn, oracle):
+    """3 -> 64 planes, 112 x 112, 3 x 3, pad 1, tiles of 16 (the shape the fused kernels are for): output and
+    gradWeight against the oracle on a slice of the planes, everything against the three-kernel tiled module,
+    and twice in a row (the second call finds the plan's buffers as the first left them)."""
+    B, P, F, k, H, pad = 4, 3, 64, 3, 112, 1
+    x, w, bias, g = _tensors(B, P, F, k, k, H, H, pad, pad, 1979)
+    fused = nn.SpatialConvolutionFFTTiledIterated(P, F, k, k, 1, 1, pad, pad, 16, 16)
+    plain = nn.SpatialConvolutionFFTTiled(P, F, k, k, 1, 1, pad, pad, 16, 16)
+    b = _three_passes(plain, x, w, bias, g, 0.25)
+    fused.weight.copy_(dev(w))
+    fused.bias.copy_(dev(bias))
+    xd, gd = dev(x), dev(g)
+    for _ in range(2):
+        fused.gradWeight.fill_(float("nan"))
+        out = host(fused.updateOutput(xd))
+        gin = host(fused.updateGradInput(xd, gd))
+        fused.accGradParameters(xd, gd, 0.25)
+        a = (out, gin, host(fused.gradWeight), host(fused.gradBias))
+        for got, want, what in zip(a, b, ("output", "gradInput", "gradWeight", "gradBias")):
+            _close(got, want, what)
+    fused.cleanupBuffers()
+    p4 = (pad,) * 4
+    fs = [0, 31, 32, 63]
+    _close(a[0][:, fs], oracle.bias_update_output(oracle.cross_correlation_valid(x, w[fs], (1, 1), p4), bias[fs]), "output")
+    _close(a[2][fs], oracle.cross_correlation_reverse_valid(x, g[:, fs], (1, 1), 0.25, p4), "gradWeight")
+    _close(a[1], oracle.convolution_full(g, w, (1, 1), p4), "gradInput")
