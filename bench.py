@@ -383,6 +383,38 @@ def measure_tiled(nn, torch, synth, steps, warmup):
     return out
 
 
+def measure_iterated(nn, torch, synth, steps):
+    """First- and last-layer shapes (few planes on one side; batch 64, 112 x 112, 3 x 3, pad 1, tiles of 16)
+    through the three-kernel tiled module and through nn.SpatialConvolutionFFTTiledIterated, whose passes are
+    single fused kernels that never write a spectrum of a feature map to memory: ms per pass, both ways."""
+    out = {}
+    passes = ("fprop", "bprop", "accgrad")
+    for name, (B, P, F, k, H, pad, tile) in {"first_layer_b64_3to64_112x112_k3_p1_tile16": (64, 3, 64, 3, 112, 1, 16),
+                                             "last_layer_b64_64to3_112x112_k3_p1_tile16": (64, 64, 3, 3, 112, 1, 16),
+                                             "mid_layer_b64_16to64_112x112_k3_p1_tile16": (64, 16, 64, 3, 112, 1, 16)}.items():
+        o = H + 2 * pad - k + 1
+        x = torch.from_numpy(synth.uniform(1007, (B, P, H, H), stream=0)).cuda()
+        g = torch.from_numpy(synth.uniform(1007, (B, F, o, o), stream=3)).cuda()
+        w = torch.from_numpy(synth.normal(1007, (F, P, k, k), 0.0, 0.05, stream=1)).cuda()
+        rec = {"gflop_per_pass": 2.0 * B * F * P * o * o * k * k / 1e9}
+        for label, cls in (("tiled_three_kernels", "SpatialConvolutionFFTTiled"), ("iterated_fused", "SpatialConvolutionFFTTiledIterated")):
+            net = getattr(nn, cls)(P, F, k, k, 1, 1, pad, pad, tile, tile)
+            net.weight.copy_(w)
+            net.bias.zero_()
+            n = max(5, steps // 3)
+            per = {p: time_loop(torch, lambda: run_pass(net, x, g, p), n, 2) for p in passes}
+            kernels = {}
+            for p in passes:
+                run_pass(net, x, g, p)
+                kernels[p] = net.stageKernels(x).get("mm", "")
+            rec[label] = {"ms_per_pass": per, "ms_per_step": sum(per.values()), "contraction_kernel": kernels}
+            net.cleanupBuffers()
+        rec["speedup_per_pass"] = {p: rec["tiled_three_kernels"]["ms_per_pass"][p] / rec["iterated_fused"]["ms_per_pass"][p]
+                                   for p in passes}
+        out[name] = rec
+    return out
+
+
 def measure_backward_step(nn, torch, synth, steps, warmup):
     """The training step as a module user runs it: updateOutput, then backward(), whose two gradient
     passes share FFT(gradOutput) (5 forward transforms per step instead of 6)."""
@@ -648,6 +680,7 @@ def main():
     if args.all_configs:
         line["other_workloads"] = {
             "tiled_convolution": measure_tiled(nn, torch, synth, args.steps, args.warmup),
+            "iterated_convolution": measure_iterated(nn, torch, synth, args.steps),
             "reference_benchmark_layers": measure_reference_list(nn, torch, synth, args.steps),
             "fft_1d": measure_fft_1d(nn, torch, args.steps, args.warmup)}
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)

@@ -81,6 +81,7 @@ struct FusedJob {
     float alpha;
     int s_off;             // LDS float offset of S; the tables sit behind it
     int tbl_off;
+    int s_alias;           // S lies in region 0 (chunked small side: it is consumed before region 0 is used again)
 };
 
 // Window table: entry j describes virtual plane (tile vb_first + j / div, plane c0 + j % div); entries
@@ -400,6 +401,7 @@ __global__ __launch_bounds__(256, (N >= 32 ? 1 : 2)) void fused_conv_kernel(Fuse
                         float re[N], im[N];
                         const int count = nvb * ns;
                         fused_forward<N>(smem, jb.small, tbl_s, count, jb.ss, tid, re, im);
+                        if (jb.s_alias) __syncthreads();  // every column has left the tile S is about to overwrite
                         if (t < count) store_column_to_S<N>(Sbuf + t * S::SPLANE, kx, re, im);
                         __syncthreads();
                     }
@@ -684,10 +686,19 @@ static hipError_t launch_fused_conv_n(FusedJob jb, int wreg_ok, hipStream_t s)
         jb.SB = T / jb.VBF;
         jb.nsc = (jb.Ns + jb.SB - 1) / jb.SB;
         s_planes = (size_t)jb.VBF * jb.SB;
+        jb.s_alias = 1;
     }
     jb.ngroups = (jb.vbatch + jb.VBF - 1) / jb.VBF;
-    jb.s_off = (int)r0;
-    jb.tbl_off = (int)(r0 + s_planes * S::SPLANE * 2);
+    if (jb.s_alias) {
+        // each chunk's spectra are multiplied before the next transform or the inverse touches region 0:
+        // S shares it, and two workgroups fit a CU
+        jb.s_off = 0;
+        const size_t sfl = s_planes * S::SPLANE * 2;
+        jb.tbl_off = (int)(sfl > r0 ? sfl : r0);
+    } else {
+        jb.s_off = (int)r0;
+        jb.tbl_off = (int)(r0 + s_planes * S::SPLANE * 2);
+    }
     jb.tbl_off = (jb.tbl_off + 3) & ~3;
     const size_t lds = (size_t)jb.tbl_off * sizeof(float) + 2 * T * sizeof(int4);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
@@ -758,9 +769,9 @@ int fused_accgrad_ranges(int N, int vbatch, int out_planes, int in_planes)
     const int nb = out_planes > in_planes ? out_planes : in_planes;
     const int ns = out_planes > in_planes ? in_planes : out_planes;
     const long blocks = (long)((nb + T - 1) / T) * ((ns + pca - 1) / pca);
-    long r = 1024 / blocks;  // about four workgroups per CU
+    long r = 512 / blocks;  // two workgroups per CU, which is what the registers allow
     if (r < 1) r = 1;
-    if (r > 64) r = 64;
+    if (r > 512) r = 512;
     if (r > vbatch) r = vbatch;
     return (int)r;
 }

@@ -76,9 +76,14 @@ class SpatialConvolution:
         for t in tiles:
             for reuse in (reuse_none, reuse_all):
                 cands.append(("SpatialConvolutionFFTTiled", t, reuse))
+        # the fused kernels keep the spectra on chip and sum over the contracted planes on the vector ALUs:
+        # a candidate where one side has few planes (first and last layers)
+        if min(self.inputPlanes, self.outputPlanes) <= 8:
+            for t in tiles:
+                cands.append(("SpatialConvolutionFFTTiledIterated", t, reuse_none))
         return cands
 
-    def _plan_bytes(self, batch, iH, iW, tile, reuse):
+    def _plan_bytes(self, batch, iH, iW, tile, reuse, cls=""):
         """Frequency-buffer bytes the strategy would allocate, or None if it cannot run."""
         kw = dict(batch=batch, in_planes=self.inputPlanes, out_planes=self.outputPlanes, in_h=iH, in_w=iW,
                   k_h=self.kH, k_w=self.kW, stride_h=self.dH, stride_w=self.dW, pad_h=self.padUp,
@@ -87,6 +92,8 @@ class SpatialConvolution:
             info = _lib.plan_query(tile_h=tile or 0, tile_w=tile or 0, **kw)
         except _lib.FbfcError:
             return None
+        if cls.endswith("Iterated"):
+            return info.weight_freq_bytes       # the fused passes own the weight spectrum only
         sizes = (info.input_freq_bytes, info.weight_freq_bytes, info.output_freq_bytes)
         # + the result buffer of a reuse policy, + what backward() adds (training only)
         return (sum(sizes) + (max(sizes) if reuse != nn.SpatialConvolutionFFT.memoryReuseNone else 0)
@@ -98,6 +105,8 @@ class SpatialConvolution:
             inst = nn.SpatialConvolutionDirect(*args, device=self.device, init=False)
         elif tile is None:
             inst = getattr(nn, cls)(*args, reuse, device=self.device)
+        elif cls.endswith("Iterated"):
+            inst = getattr(nn, cls)(*args, tile, tile, device=self.device)
         else:
             inst = getattr(nn, cls)(*args, tile, tile, reuse, device=self.device)
         inst.weight, inst.bias = self.weight, self.bias
@@ -110,7 +119,7 @@ class SpatialConvolution:
         best, best_ms = None, float("inf")
         self.timings = {}
         for cls, tile, reuse in self._candidates(iH, iW):
-            nbytes = 0 if cls == "SpatialConvolutionDirect" else self._plan_bytes(B, iH, iW, tile, reuse)
+            nbytes = 0 if cls == "SpatialConvolutionDirect" else self._plan_bytes(B, iH, iW, tile, reuse, cls)
             key = (cls, tile, reuse)
             if nbytes is None:
                 self.timings[key] = None          # the strategy cannot run this layer
