@@ -67,7 +67,9 @@ def test_backward_replays_from_a_graph(B, P, F, k, H, pad):
     assert net.prepareBackward(x) is True
     step()
     torch.cuda.synchronize()
-    assert "cgemm_backward_kernel" in net.stageKernels(x)["mm"]   # the one-grid-per-stage form ran
+    if B == 64:   # shapes the tile kernels take run both contractions as one grid
+        assert "cgemm_backward_kernel" in net.stageKernels(x)["mm"]
+    assert ";" not in net.stageKernels(x)["ifft"]   # both inverse transforms in one launch: the one-grid-per-stage form ran
     want = [host(t).copy() for t in results()]
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
