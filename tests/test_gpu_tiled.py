@@ -215,3 +215,46 @@ def test_iterated_first_layer_112(nn, oracle):
     _close(a[0][:, fs], oracle.bias_update_output(oracle.cross_correlation_valid(x, w[fs], (1, 1), p4), bias[fs]), "output")
     _close(a[2][fs], oracle.cross_correlation_reverse_valid(x, g[:, fs], (1, 1), 0.25, p4), "gradWeight")
     _close(a[1], oracle.convolution_full(g, w, (1, 1), p4), "gradInput")
+
+
+def test_iterated_backward_and_graph_replay(nn):
+    """backward() on the fused module runs its two passes one after the other (same bits as the separate calls),
+    and the three fused passes can be captured into a graph: they allocate nothing and use no memset."""
+    B, P, F, k, H, pad = 3, 3, 40, 3, 30, 1
+    x, w, bias, g = _tensors(B, P, F, k, k, H, H, pad, pad, 2024)
+    net = nn.SpatialConvolutionFFTTiledIterated(P, F, k, k, 1, 1, pad, pad, 16, 16)
+    net.weight.copy_(dev(w))
+    net.bias.copy_(dev(bias))
+    xd, gd = dev(x), dev(g)
+
+    def step():
+        net.updateOutput(xd)
+        net.updateGradInput(xd, gd)
+        net.accGradParameters(xd, gd, 0.5)
+
+    results = lambda: [net.output, net.gradInput, net.gradWeight, net.gradBias]
+    step()
+    torch.cuda.synchronize()
+    want = [host(t).copy() for t in results()]
+    for t in results()[1:]:
+        t.fill_(float("nan"))
+    net.backward(xd, gd, 0.5)
+    for got, ref, name in zip(results()[1:], want[1:], ("gradInput", "gradWeight", "gradBias")):
+        assert np.array_equal(host(got), ref), name
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        for t in results():
+            t.fill_(float("nan"))
+        (xd * 2).sum().item()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref, name in zip(results(), want, ("output", "gradInput", "gradWeight", "gradBias")):
+            assert np.array_equal(host(got), ref), "replay %d: %s differs from the eager result" % (rep, name)
+    net.cleanupBuffers()
