@@ -489,6 +489,61 @@ def measure_reference_list(nn, torch, synth, steps):
     return out
 
 
+def measure_vendor(nn, torch, synth, names, steps):
+    """The same layers through the platform library's convolution (MIOpen behind aten::convolution, fp32, with its
+    search for the fastest algorithm switched on) beside this library's time for them: the role cuDNN has in the
+    reference's benchmark (test/test_FFT.lua:300-336).  Step = updateOutput + updateGradInput + accGradParameters
+    as three calls, as in the headline; fprop_plus_backward = updateOutput + one call that produces both gradients."""
+    from fbcunn_amd.vendor import SpatialConvolutionMIOpen
+    out = {}
+    was = torch.backends.cudnn.benchmark
+    torch.backends.cudnn.benchmark = True
+    try:
+        for name in names:
+            cfg = CONFIGS[name]
+            B, P, F, H, k, pad = cfg[:6]
+            o = H + 2 * pad - k + 1
+            passes = cfg[6]
+            net, x, g = make_layer(nn, torch, synth, cfg)
+            ven = SpatialConvolutionMIOpen(P, F, k, k, 1, 1, pad, pad, init=False)
+            ven.weight, ven.bias = net.weight, net.bias
+            t0 = time.perf_counter()
+            try:
+                for p in passes:
+                    run_pass(ven, x, g, p)      # the library searches and builds its kernels here
+                torch.cuda.synchronize()
+            except RuntimeError as err:
+                out[name] = {"error": str(err)[:200]}
+                net.cleanupBuffers()
+                continue
+            first_s = time.perf_counter() - t0
+            a, b = net.updateOutput(x), ven.updateOutput(x)
+            agree = float((a - b).abs().max()) / float(b.abs().max())
+            n = max(steps, 200) if H < 32 else max(steps // 2, 10)
+            def step(mod):
+                for p in passes:
+                    run_pass(mod, x, g, p)
+            rec = {"first_call_s": first_s, "steps": n, "output_max_diff_over_max": agree,
+                   "vendor_ms_per_step": time_loop(torch, lambda: step(ven), n, max(2, n // 10)),
+                   "ms_per_step": time_loop(torch, lambda: step(net), n, max(2, n // 10))}
+            if len(passes) == 3:
+                def fb(mod):
+                    mod.updateOutput(x)
+                    mod.backward(x, g, 1.0)
+                rec["vendor_ms_fprop_plus_backward"] = time_loop(torch, lambda: fb(ven), n, max(2, n // 10))
+                rec["ms_fprop_plus_backward"] = time_loop(torch, lambda: fb(net), n, max(2, n // 10))
+            flop = len(passes) * 2.0 * B * F * P * o * o * k * k
+            rec["vendor_effective_tflops"] = flop / (rec["vendor_ms_per_step"] * 1e-3) / 1e12
+            rec["effective_tflops"] = flop / (rec["ms_per_step"] * 1e-3) / 1e12
+            rec["speedup"] = rec["vendor_ms_per_step"] / rec["ms_per_step"]
+            out[name] = rec
+            net.cleanupBuffers()
+            ven.cleanupBuffers()
+    finally:
+        torch.backends.cudnn.benchmark = was
+    return out
+
+
 def measure_spectrum_store_policy(nn, torch, synth, steps, warmup):
     """The forward transforms write their spectra through to the memory side, whose cache keeps them for the
     contraction; non-temporal stores stream them past it.  Measured alone the transform is as fast either way,
@@ -603,6 +658,8 @@ def main():
     ap.add_argument("--all-configs", action="store_true",
                     help="also measure the tiled VGG-like layer and the reference's benchmark layers")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--no-vendor", action="store_true",
+                    help="skip the platform library's convolution (its first call on a layer takes 10 s to 2 min)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run a plain 256 MiB device copy 3 times (a kernel of known traffic "
                          "for scaling FETCH_SIZE / WRITE_SIZE counter readings)")
@@ -721,6 +778,11 @@ def main():
             "iterated_convolution": measure_iterated(nn, torch, synth, args.steps),
             "reference_benchmark_layers": measure_reference_list(nn, torch, synth, args.steps),
             "fft_1d": measure_fft_1d(nn, torch, args.steps, args.warmup)}
+    if not args.no_vendor:
+        # last of the GPU work: the library's search must not sit between the measurements above.  The default run
+        # takes the headline layer only; the others' first calls take minutes
+        line["vendor_convolution"] = measure_vendor(nn, torch, synth, list(CONFIGS) if args.all_configs else [MAIN],
+                                                    args.steps)
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)
     print(json.dumps(line))
 

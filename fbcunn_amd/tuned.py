@@ -3,7 +3,8 @@ that, on the first updateOutput, times the strategies that fit the layer and kee
 fastest (:188-422).  Candidates: the FFT modules (untiled, tiles of 16 and 32, with and
 without memory reuse) and the direct convolution, which stands where the reference has
 cuDNN: it runs every layer (strides above 1, sizes no transform covers) and it is what
-the winner is checked against after tuning (:387-399), to the reference's 2e-5.
+the winner is checked against after tuning (:387-399), to the reference's 2e-5.  With
+vendor=True the platform library's convolution (MIOpen) is timed as one more candidate.
 """
 import time
 
@@ -11,6 +12,7 @@ import torch
 
 from . import _lib
 from . import modules as nn
+from . import vendor as vendor_mod
 
 __all__ = ["SpatialConvolution"]
 
@@ -38,12 +40,13 @@ class SpatialConvolution:
     directTimingFlops = 20e9
 
     def __init__(self, nInputPlane, nOutputPlane, kW, kH, dW=1, dH=1, padLeft=0, padUp=0,
-                 maximalMemoryOverhead=None, inferenceOnly=False, device="cuda"):
+                 maximalMemoryOverhead=None, inferenceOnly=False, device="cuda", vendor=False):
         self.inputPlanes, self.outputPlanes = nInputPlane, nOutputPlane
         self.kW, self.kH, self.dW, self.dH = kW, kH, dW, dH
         self.padLeft, self.padUp = padLeft, padUp
         self.maximalMemoryOverhead = maximalMemoryOverhead
         self.inferenceOnly = bool(inferenceOnly)
+        self.vendor = bool(vendor)
         self.reportLevel = 0
         self.device = torch.device(device)
         # after tuning, run the winning FFT strategy against the direct convolution (the reference
@@ -65,10 +68,12 @@ class SpatialConvolution:
     # -- candidates (SpatialConvolution.lua:237-300) -----------------------------------
     def _candidates(self, iH, iW):
         reuse_all, reuse_none = nn.SpatialConvolutionFFT.memoryReuseAll, nn.SpatialConvolutionFFT.memoryReuseNone
-        direct = ("SpatialConvolutionDirect", None, reuse_none)
+        direct = [("SpatialConvolutionDirect", None, reuse_none)]
+        if self.vendor:
+            direct.append(("SpatialConvolutionMIOpen", None, reuse_none))
         if self.dW != 1 or self.dH != 1:
-            return [direct]         # "fft only supports stride-1 convolutions atm"
-        cands = [direct, ("SpatialConvolutionFBFFT", None, reuse_all), ("SpatialConvolutionFBFFT", None, reuse_none)]
+            return direct           # "fft only supports stride-1 convolutions atm"
+        cands = direct + [("SpatialConvolutionFBFFT", None, reuse_all), ("SpatialConvolutionFBFFT", None, reuse_none)]
         if self.kH <= 9 and self.kW <= 9:
             tiles = (16, 32)
         else:
@@ -103,6 +108,8 @@ class SpatialConvolution:
         args = (self.inputPlanes, self.outputPlanes, self.kW, self.kH, self.dW, self.dH, self.padLeft, self.padUp)
         if cls == "SpatialConvolutionDirect":
             inst = nn.SpatialConvolutionDirect(*args, device=self.device, init=False)
+        elif cls == "SpatialConvolutionMIOpen":
+            inst = vendor_mod.SpatialConvolutionMIOpen(*args, device=self.device, init=False)
         elif tile is None:
             inst = getattr(nn, cls)(*args, reuse, device=self.device)
         elif cls.endswith("Iterated"):
@@ -119,7 +126,8 @@ class SpatialConvolution:
         best, best_ms = None, float("inf")
         self.timings = {}
         for cls, tile, reuse in self._candidates(iH, iW):
-            nbytes = 0 if cls == "SpatialConvolutionDirect" else self._plan_bytes(B, iH, iW, tile, reuse, cls)
+            spatial = cls in ("SpatialConvolutionDirect", "SpatialConvolutionMIOpen")
+            nbytes = 0 if spatial else self._plan_bytes(B, iH, iW, tile, reuse, cls)
             key = (cls, tile, reuse)
             if nbytes is None:
                 self.timings[key] = None          # the strategy cannot run this layer
@@ -140,7 +148,9 @@ class SpatialConvolution:
                 if not self.inferenceOnly:
                     t2 = factor * _time_function(inst.updateGradInput, x_t, g_t)
                     t3 = factor * _time_function(inst.accGradParameters, x_t, g_t, 1.0)
-            except _lib.FbfcError as err:
+            except (_lib.FbfcError, RuntimeError) as err:
+                if cls != "SpatialConvolutionMIOpen" and not isinstance(err, _lib.FbfcError):
+                    raise
                 if self.reportErrors:
                     print("%s tile %s: %s" % (cls, tile, err))
                 inst.cleanupBuffers()
@@ -157,7 +167,9 @@ class SpatialConvolution:
         if best is None:
             raise _lib.FbfcError(_lib.ERR_UNSUPPORTED_SIZE, "no strategy can run this layer")
         # correctness check of an FFT winner against the direct convolution, on random data
-        if self.selfCheck and not isinstance(best, nn.SpatialConvolutionDirect):
+        if self.selfCheck and isinstance(best, vendor_mod.SpatialConvolutionMIOpen):
+            self._check_vendor(best, input, grad_output)
+        elif self.selfCheck and not isinstance(best, nn.SpatialConvolutionDirect):
             best.cudnnDebug, best.cudnnChecks = True, True
             x = torch.randn_like(input)
             g = torch.randn_like(grad_output)
@@ -170,6 +182,26 @@ class SpatialConvolution:
                 best.cleanupBuffers()
                 raise _lib.FbfcError(_lib.ERR_HIP, "self-check of %s against the direct convolution failed" % (self.bestKey,))
         return best, best_ms
+
+    def _check_vendor(self, best, input, grad_output):
+        """The library's results against the direct convolution on random data, to the tolerance the FFT
+        modules' own check uses."""
+        ref = self._make("SpatialConvolutionDirect", None, None)
+        ref.gradWeight, ref.gradBias = torch.empty_like(self.gradWeight), torch.empty_like(self.gradBias)
+        x = torch.randn_like(input)
+        g = torch.randn_like(grad_output)
+        pairs = [(best.updateOutput(x), ref.updateOutput(x))]
+        if not self.inferenceOnly:
+            pairs.append((best.updateGradInput(x, g), ref.updateGradInput(x, g)))
+            best.accGradParameters(x, g, 1.0)
+            ref.accGradParameters(x, g, 1.0)
+            pairs.append((best.gradWeight, ref.gradWeight))
+            pairs.append((best.gradBias, ref.gradBias))
+        for got, want in pairs:
+            want = want.double()
+            err = float((want - got.double()).norm()) / (float(want.norm()) + 1e-8)
+            if not (bool(torch.isfinite(got).all()) and err <= nn.SpatialConvolutionFFT.prec):
+                raise _lib.FbfcError(_lib.ERR_HIP, "self-check of the vendor convolution against the direct one failed")
 
     def _tune(self, input):
         B, _, iH, iW = input.shape

@@ -167,3 +167,63 @@ def test_self_check_hook(fbnn):
         assert float(bad.gradBias.min()) == -2.0 == float(bad.gradBias.max())
     finally:
         nn.SpatialConvolutionFFT.prec = old
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4, 3, 3, 13, 15, 1, 1, 1, 1), (3, 2, 5, 5, 4, 23, 18, 3, 2, 2, 1)])
+def test_vendor_convolution_matches_oracle(oracle, shape):
+    """The platform library's convolution behind the module protocol (the place cudnn.SpatialConvolution has
+    in fbcunn/SpatialConvolution.lua:259-269) against the oracle; accGradParameters assigns."""
+    from fbcunn_amd.vendor import SpatialConvolutionMIOpen
+    B, P, F, kh, kw, H, W, sh, sw, ph, pw = shape
+    x = synth.uniform(41, (B, P, H, W), stream=0)
+    w = synth.normal(41, (F, P, kh, kw), 0.0, 0.1, stream=1)
+    bias = synth.uniform(41, (F,), -0.1, 0.1, stream=2)
+    oh, ow = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    g = synth.uniform(41, (B, F, oh, ow), stream=3)
+    net = SpatialConvolutionMIOpen(P, F, kw, kh, sw, sh, pw, ph, init=False)
+    net.weight.copy_(dev(w))
+    net.bias.copy_(dev(bias))
+    net.gradWeight.fill_(float("nan"))
+    net.gradBias.fill_(float("nan"))
+    xd, gd = dev(x), dev(g)
+    p4 = (ph, ph, pw, pw)
+    _close(host(net.updateOutput(xd)), oracle.bias_update_output(oracle.cross_correlation_valid(x, w, (sh, sw), p4), bias), "output")
+    # (what the oracle leaves out for strides that do not divide the padded extent: see the direct test above)
+    gi = oracle.convolution_full(g, w, (sh, sw), p4)
+    got = host(net.updateGradInput(xd, gd))
+    _close(got[:, :, :gi.shape[2], :gi.shape[3]], gi, "gradInput")
+    net.accGradParameters(xd, gd, 0.5)
+    want_gw = np.ascontiguousarray(oracle.cross_correlation_reverse_valid(x, g, (sh, sw), 0.5, p4)[:, :, :kh, :kw])
+    _close(host(net.gradWeight), want_gw, "gradWeight")
+    _close(host(net.gradBias), oracle.bias_acc_grad_parameters(g, 0.5), "gradBias")
+    net.gradWeight.fill_(float("nan"))
+    got2 = host(net.backward(xd, gd, 0.5))
+    assert np.array_equal(got2, got)
+    _close(host(net.gradWeight), want_gw, "gradWeight of backward()")
+
+
+def test_tuned_module_with_the_vendor_candidate(fbnn, oracle):
+    """vendor=True adds the library's convolution to the candidates; whichever wins matches the oracle and,
+    when it is the library, has passed the check against the direct convolution."""
+    B, P, F, k, H, pad = 2, 4, 3, 3, 40, 1
+    x = synth.uniform(43, (B, P, H, H), stream=0)
+    w = synth.normal(43, (F, P, k, k), 0.0, 0.05, stream=1)
+    bias = synth.uniform(43, (F,), -0.1, 0.1, stream=2)
+    g = synth.uniform(43, (B, F, H, H), stream=3)
+    net = fbnn.SpatialConvolution(P, F, k, k, 1, 1, pad, pad, vendor=True)
+    net.weight.copy_(dev(w))
+    net.bias.copy_(dev(bias))
+    xd, gd = dev(x), dev(g)
+    out = host(net.updateOutput(xd))
+    key = ("SpatialConvolutionMIOpen", None, "none")
+    assert key in net.timings and net.timings[key] is not None and len(net.timings[key]["ms"]) == 3
+    gin = host(net.updateGradInput(xd, gd))
+    net.accGradParameters(xd, gd, 1.0)
+    p4 = (pad,) * 4
+    _close(out, oracle.bias_update_output(oracle.cross_correlation_valid(x, w, (1, 1), p4), bias), "output")
+    _close(gin, oracle.convolution_full(g, w, (1, 1), p4), "gradInput")
+    _close(host(net.gradWeight), oracle.cross_correlation_reverse_valid(x, g, (1, 1), 1.0, p4), "gradWeight")
+    # without the flag the library is not among the candidates
+    plain = fbnn.SpatialConvolution(P, F, k, k, 1, 1, pad, pad)
+    assert all(c[0] != "SpatialConvolutionMIOpen" for c in plain._candidates(H, H))
+    net.cleanupBuffers()
