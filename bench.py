@@ -33,6 +33,7 @@ import argparse
 import json
 import os
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -489,6 +490,36 @@ def measure_reference_list(nn, torch, synth, steps):
     return out
 
 
+# Layers measured against the platform library on request (--vendor-layers): the tiled VGG-like layer, the first-,
+# last- and mid-layer shapes of the fused module and the reference's benchmark list, each through the module this
+# library would run it with.  name: (B, P, F, H, k, pad, passes, weight std, seed, module class, tile)
+_STEP = ("fprop", "bprop", "accgrad")
+VENDOR_LAYERS = {
+    "vgg_like_b64_64x128_112x112_k3_p1": (64, 64, 128, 112, 3, 1, _STEP, 0.05, 1006, "SpatialConvolutionFFTTiled", 32),
+    "first_layer_b64_3to64_112x112_k3_p1": (64, 3, 64, 112, 3, 1, _STEP, 0.05, 1007, "SpatialConvolutionFFTTiledIterated", 16),
+    "last_layer_b64_64to3_112x112_k3_p1": (64, 64, 3, 112, 3, 1, _STEP, 0.05, 1007, "SpatialConvolutionFFTTiledIterated", 16),
+    "mid_layer_b64_16to64_112x112_k3_p1": (64, 16, 64, 112, 3, 1, _STEP, 0.05, 1007, "SpatialConvolutionFFTTiled", 16),
+    "b128_96to256_24x24_k5_p2": (128, 96, 256, 24, 5, 2, _STEP, 0.05, 7, "SpatialConvolutionFBFFT", None),
+    "b128_256to512_12x12_k3_p1": (128, 256, 512, 12, 3, 1, _STEP, 0.05, 7, "SpatialConvolutionFBFFT", None),
+    "b128_512to1024_12x12_k3_p1": (128, 512, 1024, 12, 3, 1, _STEP, 0.05, 7, "SpatialConvolutionFBFFT", None),
+    "b128_1024to1024_12x12_k3_p1": (128, 1024, 1024, 12, 3, 1, _STEP, 0.05, 7, "SpatialConvolutionFBFFT", None),
+}
+
+
+def make_vendor_layer(nn, torch, synth, name):
+    if name in CONFIGS:
+        return make_layer(nn, torch, synth, CONFIGS[name])
+    B, P, F, H, k, pad, _, wstd, seed, cls, tile = VENDOR_LAYERS[name]
+    o = H + 2 * pad - k + 1
+    args = (P, F, k, k, 1, 1, pad, pad) + ((tile, tile) if tile else ())
+    net = getattr(nn, cls)(*args)
+    net.weight.copy_(torch.from_numpy(synth.normal(seed, (F, P, k, k), 0.0, wstd, stream=1)).cuda())
+    net.bias.copy_(torch.from_numpy(synth.uniform(seed, (F,), -0.1, 0.1, stream=2)).cuda())
+    x = torch.from_numpy(synth.uniform(seed, (B, P, H, H), stream=0)).cuda()
+    g = torch.from_numpy(synth.uniform(seed, (B, F, o, o), stream=3)).cuda()
+    return net, x, g
+
+
 def measure_vendor(nn, torch, synth, names, steps):
     """The same layers through the platform library's convolution (MIOpen behind aten::convolution, fp32, with its
     search for the fastest algorithm switched on) beside this library's time for them: the role cuDNN has in the
@@ -500,18 +531,30 @@ def measure_vendor(nn, torch, synth, names, steps):
     torch.backends.cudnn.benchmark = True
     try:
         for name in names:
-            cfg = CONFIGS[name]
+            cfg = CONFIGS[name] if name in CONFIGS else VENDOR_LAYERS[name]
             B, P, F, H, k, pad = cfg[:6]
             o = H + 2 * pad - k + 1
             passes = cfg[6]
-            net, x, g = make_layer(nn, torch, synth, cfg)
+            net, x, g = make_vendor_layer(nn, torch, synth, name)
+            print("bench.py: platform library on %s (its search can take minutes)" % name, file=sys.stderr, flush=True)
             ven = SpatialConvolutionMIOpen(P, F, k, k, 1, 1, pad, pad, init=False)
             ven.weight, ven.bias = net.weight, net.bias
             t0 = time.perf_counter()
+            # a line a minute while the library searches, for whoever watches the run
+            done = threading.Event()
+            def heartbeat():
+                while not done.wait(60.0):
+                    print("bench.py: ... still searching (%d s)" % (time.perf_counter() - t0), file=sys.stderr, flush=True)
+            beat = threading.Thread(target=heartbeat, daemon=True)
+            beat.start()
             try:
-                for p in passes:
-                    run_pass(ven, x, g, p)      # the library searches and builds its kernels here
-                torch.cuda.synchronize()
+                try:
+                    for p in passes:
+                        run_pass(ven, x, g, p)      # the library searches and builds its kernels here
+                    torch.cuda.synchronize()
+                finally:
+                    done.set()
+                    beat.join()
             except RuntimeError as err:
                 out[name] = {"error": str(err)[:200]}
                 net.cleanupBuffers()
@@ -523,7 +566,7 @@ def measure_vendor(nn, torch, synth, names, steps):
             def step(mod):
                 for p in passes:
                     run_pass(mod, x, g, p)
-            rec = {"first_call_s": first_s, "steps": n, "output_max_diff_over_max": agree,
+            rec = {"module": type(net).__name__, "first_call_s": first_s, "steps": n, "output_max_diff_over_max": agree,
                    "vendor_ms_per_step": time_loop(torch, lambda: step(ven), n, max(2, n // 10)),
                    "ms_per_step": time_loop(torch, lambda: step(net), n, max(2, n // 10))}
             if len(passes) == 3:
@@ -660,6 +703,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-vendor", action="store_true",
                     help="skip the platform library's convolution (its first call on a layer takes 10 s to 2 min)")
+    ap.add_argument("--vendor-layers", action="store_true",
+                    help="also time the tiled, first-/last-layer and reference-benchmark layers against the platform "
+                         "library (its searches add about 12 minutes)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run a plain 256 MiB device copy 3 times (a kernel of known traffic "
                          "for scaling FETCH_SIZE / WRITE_SIZE counter readings)")
@@ -781,8 +827,10 @@ def main():
     if not args.no_vendor:
         # last of the GPU work: the library's search must not sit between the measurements above.  The default run
         # takes the headline layer only; the others' first calls take minutes
-        line["vendor_convolution"] = measure_vendor(nn, torch, synth, list(CONFIGS) if args.all_configs else [MAIN],
-                                                    args.steps)
+        names = list(CONFIGS) if args.all_configs else [MAIN]
+        if args.vendor_layers:
+            names += list(VENDOR_LAYERS)
+        line["vendor_convolution"] = measure_vendor(nn, torch, synth, names, args.steps)
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)
     print(json.dumps(line))
 

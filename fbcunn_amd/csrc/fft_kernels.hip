@@ -225,10 +225,13 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
         } else {
             bool windowed = false;
             if constexpr (WIN) windowed = win.on != 0;
+            // floats between the canvases of two planes, and where the all-zero row lies
+            const int pstride = windowed ? window_plane_stride<N>(h) : h * LDR;
+            const int zoff = windowed ? S::TP * pstride : zrow * LDR;
             if (windowed) {
                 if (hs == 0) __syncthreads();  // window table complete
-                zero_canvas_margins<N, S::THREADS>(smem, 0, w, 0, zrow, tid);  // the all-zero row only
-                copy_windows<N, true>(smem, const_cast<float *>(in), tbl, hs * S::TP, nph, h, w, 0, win, tid);
+                if (tid < N) smem[zoff + tid] = 0.0f;
+                copy_windows<N, true>(smem, const_cast<float *>(in), tbl, hs * S::TP, nph, h, w, 0, win, tid, pstride);
             } else {
                 zero_canvas_margins<N, S::THREADS>(smem, nph * h, w, padL, zrow, tid);
                 copy_canvas<N, true, S::THREADS>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
@@ -236,8 +239,8 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
             __syncthreads();
             if (row_active && round_of_lane == hs) {
                 const int tl = t - hs * S::TP;
-                const float4 *pa = reinterpret_cast<const float4 *>(smem + (va ? tl * h + ia : zrow) * LDR);
-                const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? tl * h + ib : zrow) * LDR);
+                const float4 *pa = reinterpret_cast<const float4 *>(smem + (va ? tl * pstride + ia * LDR : zoff));
+                const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? tl * pstride + ib * LDR : zoff));
                 static_for<N / 4>([&](auto jj) {
                     constexpr int j = decltype(jj)::value;
                     if constexpr (4 * j < NZ) {
@@ -505,10 +508,13 @@ __global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftSh
         int nph = np - hs * S::TP;
         nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
         if (hs > 0) __syncthreads();  // previous round copied out
+        bool windowed = false;
+        if constexpr (WIN) windowed = win.on != 0;
+        const int pstride = windowed ? window_plane_stride<N>(h) : h * LDR;
         if (row_active && round_of_lane == hs) {
             const int tl = tr - hs * S::TP;
             if (va) {
-                float4 *pa = reinterpret_cast<float4 *>(smem + (tl * h + ia) * LDR);
+                float4 *pa = reinterpret_cast<float4 *>(smem + tl * pstride + ia * LDR);
                 static_for<N / 4>([&](auto jj) {
                     constexpr int j = decltype(jj)::value;
                     pa[j] = make_float4(zr[brev<N>(4 * j)] + bv, zr[brev<N>(4 * j + 1)] + bv,
@@ -516,7 +522,7 @@ __global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftSh
                 });
             }
             if (vb) {
-                float4 *pb = reinterpret_cast<float4 *>(smem + (tl * h + ib) * LDR);
+                float4 *pb = reinterpret_cast<float4 *>(smem + tl * pstride + ib * LDR);
                 static_for<N / 4>([&](auto jj) {
                     constexpr int j = decltype(jj)::value;
                     pb[j] = make_float4(zi[brev<N>(4 * j)] + bv, zi[brev<N>(4 * j + 1)] + bv,
@@ -525,10 +531,8 @@ __global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftSh
             }
         }
         __syncthreads();
-        bool windowed = false;
-        if constexpr (WIN) windowed = win.on != 0;
         if (windowed)
-            copy_windows<N, false>(smem, out, tbl, hs * S::TP, nph, h, w, padL, win, tid);
+            copy_windows<N, false>(smem, out, tbl, hs * S::TP, nph, h, w, padL, win, tid, pstride);
         else
             copy_canvas<N, false, S::THREADS>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
     });
@@ -538,7 +542,7 @@ __global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftSh
 // host launchers
 // ---------------------------------------------------------------------------------
 template <int N, bool INVERSE, bool SMALL = false, int PHASES = 0>
-static size_t fft_lds_bytes(int h, int w, int padU)
+static size_t fft_lds_bytes(int h, int w, int padU, bool windowed = false)
 {
     using S = FftShape<N, INVERSE, SMALL, PHASES>;
     (void)padU;
@@ -546,7 +550,8 @@ static size_t fft_lds_bytes(int h, int w, int padU)
     const size_t tile = (size_t)(SMALL ? 16 : N) * S::ROWSTRIDE * sizeof(float2);
     // canvas-row staging (the inverse, windowed operands, N = 128) or, smaller, the raw chunk with N
     // floats of slack on either side and N zeros behind
-    const size_t canvas = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
+    const size_t canvas = windowed ? ((size_t)S::TP * window_plane_stride<N>(h) + Canvas<N>::LDR) * sizeof(float)
+                                   : ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
     const size_t raw = ((size_t)S::TP * h * w + 3 * N) * sizeof(float);
     const size_t stage = canvas > raw ? canvas : raw;
     return ((tile > stage ? tile : stage) + 15) & ~(size_t)15;
@@ -595,19 +600,19 @@ template <int N, bool WIN, int NZ, bool RAW>
 static hipError_t launch_fwd_impl(const FwdArgs &a, const FwdArgs *second, hipStream_t s,
                                   const FwdArgs *third = nullptr)
 {
-    size_t lds = fft_lds_bytes<N, false, (NZ < N)>(a.h, a.w, a.padU);
+    size_t lds = fft_lds_bytes<N, false, (NZ < N)>(a.h, a.w, a.padU, a.win.on != 0);
     const long blocks0 = fwd_blocks<N>(a.planes);
     long blocks01 = blocks0, blocks = blocks0;
     FwdJob j0 = make_job<N, (NZ < N)>(a);
     FwdJob j1 = j0, j2 = j0;
     if (second != nullptr) {
-        const size_t lds1 = fft_lds_bytes<N, false, (NZ < N)>(second->h, second->w, second->padU);
+        const size_t lds1 = fft_lds_bytes<N, false, (NZ < N)>(second->h, second->w, second->padU, second->win.on != 0);
         if (lds1 > lds) lds = lds1;
         blocks01 += fwd_blocks<N>(second->planes);
         blocks = blocks01;
         j1 = make_job<N, (NZ < N)>(*second);
         if (third != nullptr) {
-            const size_t lds2 = fft_lds_bytes<N, false, (NZ < N)>(third->h, third->w, third->padU);
+            const size_t lds2 = fft_lds_bytes<N, false, (NZ < N)>(third->h, third->w, third->padU, third->win.on != 0);
             if (lds2 > lds) lds = lds2;
             blocks += fwd_blocks<N>(third->planes);
             j2 = make_job<N, (NZ < N)>(*third);
@@ -662,7 +667,7 @@ template <int N, bool WIN, int PHASES>
 static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s, const InvArgs *second = nullptr)
 {
     using S = FftShape<N, true, false, PHASES>;
-    size_t lds = fft_lds_bytes<N, true, false, PHASES>(a.h, a.w, a.padU);
+    size_t lds = fft_lds_bytes<N, true, false, PHASES>(a.h, a.w, a.padU, a.win.on != 0);
     auto nblocks = [](long planes) {
         long b = (planes + S::T - 1) / S::T;
         if (S::T * 8 < 128) b = (b + 15) / 16 * 16;  // whole cycles of the paired mapping
@@ -674,7 +679,7 @@ static hipError_t launch_inv_impl(const InvArgs &a, hipStream_t s, const InvArgs
     InvJob j1 = j0;
     const InvArgs *bg = (a.go_freq != nullptr) ? &a : nullptr;
     if (second != nullptr) {
-        const size_t lds1 = fft_lds_bytes<N, true, false, PHASES>(second->h, second->w, second->padU);
+        const size_t lds1 = fft_lds_bytes<N, true, false, PHASES>(second->h, second->w, second->padU, second->win.on != 0);
         if (lds1 > lds) lds = lds1;
         blocks += nblocks(second->planes);
         j1 = make_inv_job<N, WIN, PHASES>(*second);

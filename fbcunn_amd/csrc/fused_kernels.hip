@@ -119,13 +119,14 @@ __device__ __forceinline__ void fused_forward(float *smem, const float *in, cons
     const int ya = 2 * rp, yb = ya + 1;
     const bool va = ya < h, vb = yb < h;
     const bool row_active = (t < count) && (va || vb);
-    const int zrow = T * h;  // an all-zero canvas row behind the staged windows
-    if (tid < N) smem[zrow * LDR + tid] = 0.0f;
-    copy_windows<N, true>(smem, const_cast<float *>(in), tbl, 0, count, h, w, 0, sd.win, tid);
+    const int pstride = window_plane_stride<N>(h);
+    const int zoff = T * pstride;  // an all-zero canvas row behind the staged windows
+    if (tid < N) smem[zoff + tid] = 0.0f;
+    copy_windows<N, true>(smem, const_cast<float *>(in), tbl, 0, count, h, w, 0, sd.win, tid, pstride);
     __syncthreads();
     if (row_active) {
-        const float4 *pa = reinterpret_cast<const float4 *>(smem + (va ? t * h + ya : zrow) * LDR);
-        const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? t * h + yb : zrow) * LDR);
+        const float4 *pa = reinterpret_cast<const float4 *>(smem + (va ? t * pstride + ya * LDR : zoff));
+        const float4 *pb = reinterpret_cast<const float4 *>(smem + (vb ? t * pstride + yb * LDR : zoff));
         static_for<N / 4>([&](auto jj) {
             constexpr int j = decltype(jj)::value;
             const float4 a = pa[j], b = pb[j];
@@ -305,10 +306,11 @@ __device__ __forceinline__ void fused_inverse(float *smem, float *out, const int
         });
     }
     __syncthreads();  // tile consumed: the staging area may overwrite it
+    const int pstride = window_plane_stride<N>(sd.h);
     if (row_active) {
         fft_inplace<N, true>(zr, zi);
         if (va) {
-            float4 *pa = reinterpret_cast<float4 *>(smem + (t * sd.h + ia) * LDR);
+            float4 *pa = reinterpret_cast<float4 *>(smem + t * pstride + ia * LDR);
             static_for<N / 4>([&](auto jj) {
                 constexpr int j = decltype(jj)::value;
                 pa[j] = make_float4(zr[brev<N>(4 * j)] + bias_v, zr[brev<N>(4 * j + 1)] + bias_v,
@@ -316,7 +318,7 @@ __device__ __forceinline__ void fused_inverse(float *smem, float *out, const int
             });
         }
         if (vb) {
-            float4 *pb = reinterpret_cast<float4 *>(smem + (t * sd.h + ib) * LDR);
+            float4 *pb = reinterpret_cast<float4 *>(smem + t * pstride + ib * LDR);
             static_for<N / 4>([&](auto jj) {
                 constexpr int j = decltype(jj)::value;
                 pb[j] = make_float4(zi[brev<N>(4 * j)] + bias_v, zi[brev<N>(4 * j + 1)] + bias_v,
@@ -325,7 +327,7 @@ __device__ __forceinline__ void fused_inverse(float *smem, float *out, const int
         }
     }
     __syncthreads();
-    copy_windows<N, false>(smem, out, tbl, 0, T, sd.h, sd.w, sd.padL, sd.win, tid);
+    copy_windows<N, false>(smem, out, tbl, 0, T, sd.h, sd.w, sd.padL, sd.win, tid, pstride);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -651,7 +653,7 @@ static size_t fused_region0_floats(int h_small, int h_big)
     using S = FusedShape<N>;
     const size_t tile = (size_t)2 * N * S::ROWSTRIDE;
     const int h = h_small > h_big ? h_small : h_big;
-    const size_t stage = ((size_t)S::T * h + 1) * Canvas<N>::LDR;
+    const size_t stage = (size_t)S::T * (h * Canvas<N>::LDR + 4) + Canvas<N>::LDR;
     return ((tile > stage ? tile : stage) + 3) & ~(size_t)3;
 }
 
