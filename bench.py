@@ -555,8 +555,8 @@ def measure_vendor(nn, torch, synth, names, steps):
                 finally:
                     done.set()
                     beat.join()
-            except RuntimeError as err:
-                out[name] = {"error": str(err)[:200]}
+            except Exception as err:
+                out[name] = {"error": "%s: %s" % (type(err).__name__, str(err)[:200])}
                 net.cleanupBuffers()
                 continue
             first_s = time.perf_counter() - t0
@@ -830,7 +830,10 @@ def main():
         names = list(CONFIGS) if args.all_configs else [MAIN]
         if args.vendor_layers:
             names += list(VENDOR_LAYERS)
-        line["vendor_convolution"] = measure_vendor(nn, torch, synth, names, args.steps)
+        try:
+            line["vendor_convolution"] = measure_vendor(nn, torch, synth, names, args.steps)
+        except Exception as err:    # a comparison figure must not cost the line
+            line["vendor_convolution"] = {"error": "%s: %s" % (type(err).__name__, str(err)[:200])}
     line["cpu_baseline"] = None if args.no_cpu else cpu_baseline(synth)
     print(json.dumps(line))
 
