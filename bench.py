@@ -323,7 +323,7 @@ def measure_fft_1d(nn, torch, steps, warmup):
     """Batched 1-D transforms (fbfft1dHost's job, src/fft/FBFFTHost.cpp:119-131): 256 MiB of real rows
     of each size, forward and unnormalised inverse; bytes = the rows once plus the half spectra once."""
     out = {}
-    for n in (8, 32, 128):
+    for n in (8, 32, 64, 128):
         rows = (1 << 26) // n
         x = torch.rand(rows, n, device="cuda")
         freq = torch.empty((rows, n // 2 + 1, 2), device="cuda")

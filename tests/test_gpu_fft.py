@@ -176,6 +176,8 @@ def test_1d_forward_and_inverse(nn, oracle, n, rows, m, pl):
     freq = torch.full((rows, n // 2 + 1, 2), float("nan"), device="cuda")
     w = nn.FFTWrapper("fbfft", pl, 0)
     w.fft(dev(x), freq)
+    # sizes from 32 on run a row over 2, 4 or 8 lanes with cross-lane butterflies
+    assert ("rfft1d_split_kernel" in w.lastKernel()) == (n >= 32)
     got = host(freq)
     got = got[..., 0] + 1j * got[..., 1]
     scale = max(np.abs(want).max(), 1e-30)
@@ -197,7 +199,7 @@ def test_1d_forward_and_inverse(nn, oracle, n, rows, m, pl):
     assert np.abs(back - wantb).max() <= 4 * TOL * np.abs(wantb).max()
 
 
-@pytest.mark.parametrize("n", [8, 32, 128])
+@pytest.mark.parametrize("n", [8, 32, 64, 128])
 def test_1d_rows_that_do_not_start_on_16_bytes(nn, n):
     """Row lengths that are multiples of four floats take 16-byte pieces only if the tensor itself starts on
     a 16-byte boundary; a view one float into a buffer takes the 4-byte path and gives the same numbers."""
