@@ -732,7 +732,7 @@ static int splitk_override() { return g_force_variant.load(std::memory_order_rel
 //  * N a multiple of 96 but not of 64 (96 input planes): 64x32 tiles by two waves.  At 2112 frequencies
 //    256x96x64 conj(A)^T B takes 268 us (284 with 64x96 tiles by six waves, 321 with the register-fed
 //    kernel); 64x96x256 A B is as fast either way (251 us) and keeps the register-fed kernel;
-//  * at least 4 full 64x64 tiles per CU and 64-aligned M, N: LDS-direct tiles;
+//  * at least 4 full 64x64 tiles per CU, or at least one and K >= 32, and 64-aligned M, N: LDS-direct tiles;
 //  * otherwise, if M, N are multiples of 32 and K of 16: the register-fed kernel, with more
 //    waves sharing one block's K range the fewer blocks there are per SIMD;
 //  * anything else: register-staged LDS tiles with bounds checks.
@@ -760,7 +760,11 @@ static Choice choose_variant(int mode, const float *A, const float *B, int n_fre
     if ((mode != 1 || force == 8) && (m % 64) == 0 && (n % 96) == 0 && (n % 64) != 0 && (k % 16) == 0 && aligned16 &&
         (force == 8 || (force < 0 && (long)n_freq * (m / 64) * (n / 96) >= 4 * 256)))
         return {V_TILES32, 0};
-    const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && total >= 4 * 256));
+    // one to four rounds of tiles that the hybrid does not take (a last round more than half full, or none):
+    // whole tiles still beat the register-fed kernel once K is 32 or more (128^3 per frequency: 480 tiles
+    // 16.9 against 21.0 us, 512 tiles 17.3 against 21.6, 768 tiles 24.4 against 32.1, 256 tiles 11.1 against 11.9;
+    // 130 x 128x128x32: 8.5 against 10.1)
+    const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && (total >= 4 * 256 || (total >= 256 && k >= 32))));
     if (!prefer_direct && (m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 &&
         tot32 * 4 < 0x7fffff00L) {
         int sk = 0;

@@ -32,6 +32,8 @@ SHAPES = [  # Q, m, n, k
     # a few rounds of 64x64 tiles with a ragged last one: whole rounds as LDS-direct tiles, the
     # left-over frequencies as split blocks, in one launch
     (70, 128, 128, 64), (300, 64, 64, 128), (33, 192, 128, 64),
+    # one to four rounds of tiles whose last round is more than half full (or full): whole tiles throughout
+    (60, 128, 256, 128), (130, 128, 128, 32), (64, 128, 128, 128),
     # N a multiple of 96 but not of 64 and at least 1024 64x96 blocks: 64x32 tiles by two waves
     (1024, 64, 96, 16), (260, 128, 288, 32), (1100, 64, 96, 48),
 ]
@@ -91,6 +93,23 @@ def test_against_oracle_contraction(nn, oracle, pass_):
         nn.transposeMM(dev(to_fm(G)), dev(to_fm(I)), C, alpha, True, False, False)
     got = np.transpose(host(C), (1, 2, 0, 3))
     assert np.abs(got - want).max() <= TOL * np.abs(want).max()
+
+
+@pytest.mark.parametrize("shape,kernel", [((3, 128, 128, 128), "cgemm_splitk_kernel"), ((70, 128, 128, 64), "cgemm_hybrid_kernel"),
+                                          ((300, 64, 64, 128), "cgemm_hybrid_kernel"), ((60, 128, 256, 128), "cgemm_ldsdirect_kernel"),
+                                          ((130, 128, 128, 32), "cgemm_ldsdirect_kernel"), ((64, 128, 128, 128), "cgemm_ldsdirect_kernel"),
+                                          ((300, 128, 128, 64), "cgemm_ldsdirect_kernel"), ((6, 3, 5, 7), "cgemm_freq_kernel")])
+def test_which_kernel_a_shape_takes(nn, shape, kernel):
+    """The shape rule of the contraction: few tiles -> register-fed blocks with K shared by the waves; a few rounds
+    of tiles with a thin last round -> tiles plus split blocks in one launch; otherwise whole tiles; ragged sizes ->
+    the bounds-checked kernel."""
+    from fbcunn_amd import _lib
+    Q, m, n, k = shape
+    A = torch.zeros((Q, m, k, 2), device="cuda")
+    B = torch.zeros((Q, n, k, 2), device="cuda")
+    C = torch.empty((Q, m, n, 2), device="cuda")
+    nn.transposeMM(A, B, C, 1.0, False, True, False)
+    assert _lib.lib().fbfc_last_launch().decode().startswith(kernel)
 
 
 def test_both_conjugations_rejected(nn):
