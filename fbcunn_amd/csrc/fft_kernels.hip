@@ -186,7 +186,6 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
     // different LDS banks by themselves); windowed operands, even sizes (a 32 x 32 plane staged raw puts
     // every row on the same banks) and N = 128 are staged as zero-padded canvas rows.
     static_assert(!RAW || (!WIN && N <= 64), "raw staging: plain operands, N <= 64");
-    const int zrow = S::TP * h;  // canvas staging: an all-zero row for canvas rows outside the plane
     // raw staging: bit x of colmask = canvas column x lies inside the plane
     [[maybe_unused]] const unsigned long long colmask = ((w >= 64) ? ~0ull : ((1ull << w) - 1ull)) << padL;
     static_for<S::PH>([&](auto hh) {
@@ -227,13 +226,13 @@ __global__ __launch_bounds__((FftShape<N, false, (NZ < N)>::THREADS), (FftShape<
             if constexpr (WIN) windowed = win.on != 0;
             // floats between the canvases of two planes, and where the all-zero row lies
             const int pstride = windowed ? window_plane_stride<N>(h) : h * LDR;
-            const int zoff = windowed ? S::TP * pstride : zrow * LDR;
+            const int zoff = S::TP * pstride;
             if (windowed) {
                 if (hs == 0) __syncthreads();  // window table complete
                 if (tid < N) smem[zoff + tid] = 0.0f;
                 copy_windows<N, true>(smem, const_cast<float *>(in), tbl, hs * S::TP, nph, h, w, 0, win, tid, pstride);
             } else {
-                zero_canvas_margins<N, S::THREADS>(smem, nph * h, w, padL, zrow, tid);
+                zero_canvas_margins<N, S::THREADS>(smem, nph * h, w, padL, zoff, tid);
                 copy_canvas<N, true, S::THREADS>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
             }
             __syncthreads();
@@ -510,7 +509,7 @@ __global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftSh
         if (hs > 0) __syncthreads();  // previous round copied out
         bool windowed = false;
         if constexpr (WIN) windowed = win.on != 0;
-        const int pstride = windowed ? window_plane_stride<N>(h) : h * LDR;
+        const int pstride = windowed ? window_plane_stride<N>(h) : h * LDR + job.ppad;
         if (row_active && round_of_lane == hs) {
             const int tl = tr - hs * S::TP;
             if (va) {
@@ -534,7 +533,7 @@ __global__ __launch_bounds__((FftShape<N, true, false, PHASES>::THREADS), (FftSh
         if (windowed)
             copy_windows<N, false>(smem, out, tbl, hs * S::TP, nph, h, w, padL, win, tid, pstride);
         else
-            copy_canvas<N, false, S::THREADS>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
+            copy_canvas<N, false, S::THREADS>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid, h, job.ppad);
     });
 }
 
@@ -550,8 +549,9 @@ static size_t fft_lds_bytes(int h, int w, int padU, bool windowed = false)
     const size_t tile = (size_t)(SMALL ? 16 : N) * S::ROWSTRIDE * sizeof(float2);
     // canvas-row staging (the inverse, windowed operands, N = 128) or, smaller, the raw chunk with N
     // floats of slack on either side and N zeros behind
-    const size_t canvas = windowed ? ((size_t)S::TP * window_plane_stride<N>(h) + Canvas<N>::LDR) * sizeof(float)
-                                   : ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
+    // (+ 4 floats per plane: the most canvas_plane_pad asks for with these kernels' lane order)
+    const size_t canvas = ((size_t)S::TP * (h * Canvas<N>::LDR + 4) + Canvas<N>::LDR) * sizeof(float);
+    (void)windowed;
     const size_t raw = ((size_t)S::TP * h * w + 3 * N) * sizeof(float);
     const size_t stage = canvas > raw ? canvas : raw;
     return ((tile > stage ? tile : stage) + 15) & ~(size_t)15;
@@ -656,6 +656,7 @@ static InvJob make_inv_job(const InvArgs &a)
     j.bias_period = a.bias_period > 0 ? a.bias_period : 1;
     // every copy-out round starts TP planes after the previous one: all of them 16-byte aligned
     j.vec4 = ((reinterpret_cast<uintptr_t>(a.out) & 15) == 0) && (((long)S::TP * a.h * a.w) % 4 == 0);
+    j.ppad = a.win.on ? 0 : canvas_plane_pad(Canvas<N>::LDR, a.h, a.w, j.vec4, 2, 1);
     j.tbl_off = 0;
     j.win = a.win;
     j.win.remap = window_remap_ok<S::T>(a.win, a.planes);

@@ -170,7 +170,7 @@ rfft2d_rows_kernel(FwdJob job0, FwdJob job1, FwdJob job2, unsigned blocks0, unsi
                 });
             }
         } else {
-            zero_canvas_margins<N, S::THREADS>(smem, nph * h, w, padL, S::TP * h, tid);
+            zero_canvas_margins<N, S::THREADS>(smem, nph * h, w, padL, S::TP * h * LDR, tid);
             copy_canvas<N, true, S::THREADS>(smem, const_cast<float *>(in) + (x0 + hs * S::TP) * hw, nph * h, w, padL,
                                              vec4, tid);
             __syncthreads();
@@ -340,7 +340,7 @@ __device__ __forceinline__ void load_column(float (&re)[N / 2], float (&im)[N / 
 template <int N, int T>
 __global__ __launch_bounds__((RowShape<N, T>::THREADS), (RowShape<N, T>::MIN_WAVES)) void
 irfft2d_rows_kernel(const float2 *__restrict__ in, float *__restrict__ out, long planes, int h, int w, int padU,
-                    int padL, const float *__restrict__ bias, int bias_period, int vec4, BiasGradJob bgrad,
+                    int padL, const float *__restrict__ bias, int bias_period, int vec4, int ppad, BiasGradJob bgrad,
                     unsigned bgrad_blocks)
 {
     using S = RowShape<N, T>;
@@ -463,7 +463,7 @@ irfft2d_rows_kernel(const float2 *__restrict__ in, float *__restrict__ out, long
         nph = nph < 0 ? 0 : (nph > S::TP ? S::TP : nph);
         if (hs > 0) __syncthreads();  // previous round copied out
         if (row_active && round_of_lane == hs) {
-            float4 *p = reinterpret_cast<float4 *>(smem + ((tr - hs * S::TP) * h + iy) * LDR);
+            float4 *p = reinterpret_cast<float4 *>(smem + (tr - hs * S::TP) * (h * LDR + ppad) + iy * LDR);
             static_for<N / 4>([&](auto jj) {
                 constexpr int j = decltype(jj)::value;
                 p[j] = make_float4(zr[brev<M>(2 * j)] + bv, zi[brev<M>(2 * j)] + bv,
@@ -471,7 +471,7 @@ irfft2d_rows_kernel(const float2 *__restrict__ in, float *__restrict__ out, long
             });
         }
         __syncthreads();
-        copy_canvas<N, false, S::THREADS>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid);
+        copy_canvas<N, false, S::THREADS>(smem, out + (x0 + hs * S::TP) * hw, nph * h, w, padL, vec4, tid, h, ppad);
     });
 }
 
@@ -483,10 +483,20 @@ static size_t rows_lds_bytes(int h, int w)
 {
     using S = RowShape<N, T, SMALL>;
     const size_t tile = (size_t)(SMALL ? 16 : N) * S::ROWSTRIDE * sizeof(float2);
-    const size_t canvas = ((size_t)S::TP * h + 1) * Canvas<N>::LDR * sizeof(float);
+    // (+ up to 4 (32 / TP - 1) floats per plane: canvas_plane_pad with this kernel's lane order)
+    const size_t canvas = ((size_t)S::TP * (h * Canvas<N>::LDR + 4 * (32 / S::TP - 1)) + Canvas<N>::LDR) * sizeof(float);
     const size_t raw = ((size_t)S::TP * h * w + 3 * N) * sizeof(float);
     const size_t stage = canvas > raw ? canvas : raw;
     return ((tile > stage ? tile : stage) + 15) & ~(size_t)15;
+}
+
+// one row per lane, TP planes fastest: 16 lanes are TP planes times 16 / TP consecutive rows
+template <int TP>
+static int rows_plane_pad(int ldr, int h, int w, int vec4)
+{
+    static_assert(TP == 2 || TP == 4 || TP == 8 || TP == 16, "planes per staging round");
+    if (TP == 16) return canvas_plane_pad(ldr, h, w, vec4, 2, 1);
+    return canvas_plane_pad(ldr, h, w, vec4, 32 / TP, 16 / TP);
 }
 
 template <int N, int T, bool SMALL>
@@ -559,9 +569,10 @@ static hipError_t launch_inv_rows(const InvArgs &a, hipStream_t s)
         snprintf(name, sizeof name, "irfft2d_rows_kernel<%d, %d>", N, T);
         kernel_log_add(name, (blocks + bblocks) * S::THREADS);
     }
+    const int ppad = rows_plane_pad<S::TP>(Canvas<N>::LDR, a.h, a.w, vec4);
     FBFC_LAUNCH((irfft2d_rows_kernel<N, T>), dim3((unsigned)blocks + bblocks), dim3(S::THREADS), lds, s,
                        reinterpret_cast<const float2 *>(a.in), a.out, a.planes, a.h, a.w, a.padU, a.padL, a.bias,
-                       a.bias_period > 0 ? a.bias_period : 1, vec4, bgrad, bblocks);
+                       a.bias_period > 0 ? a.bias_period : 1, vec4, ppad, bgrad, bblocks);
     return hipGetLastError();
 }
 

@@ -44,9 +44,13 @@ inline long plane_group_blocks(long planes)
     return blocks;
 }
 
+// Global -> canvas rows (forward transforms): nrows rows of w floats, contiguous in memory, to rows of LDR floats.
+// Canvas rows -> global (inverse transforms): the reverse.  ppad > 0 (inverse only): the canvases of consecutive
+// planes (h rows each) lie ppad floats further apart than their rows alone (canvas_plane_pad); only with 16-byte
+// pieces and planes of a multiple of four floats, so that a piece never straddles two planes.
 template <int N, bool TO_LDS, int NT = 256>
 __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, int w, int padL,
-                                            int vec4, int tid)
+                                            int vec4, int tid, int h = 1, int ppad = 0)
 {
     constexpr int LDR = Canvas<N>::LDR;
     const int total = nrows * w;
@@ -95,18 +99,55 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
                 }
             }
         } else {
-            for (int i = tid; i < n4; i += NT) {
-                float v[4];
-                int r_ = row, x_ = x;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    v[c] = smem[r_ * LDR + padL + x_];
-                    if (++x_ == w) { x_ = 0; ++r_; }
+            if ((w & 1) == 0) {
+                // Even widths: the two halves of a 16-byte piece lie in one canvas row each, so a piece costs two
+                // addresses instead of four with a wrap test per element, and 8-byte LDS reads when the padding
+                // is even too.  pl, pe: plane of the lane's piece and the piece's first element within it.
+                const int hw = h * w;
+                int pl = 0, pe = 0, dpl = 0, dpe = 0;
+                if (ppad) {
+                    pl = (tid * 4) / hw;
+                    pe = tid * 4 - pl * hw;
+                    dpl = (4 * NT) / hw;
+                    dpe = 4 * NT - dpl * hw;
                 }
-                store_nt(g4 + i, make_float4(v[0], v[1], v[2], v[3]));
-                row += drow;
-                x += dx;
-                if (x >= w) { x -= w; ++row; }
+                const bool even_pad = (padL & 1) == 0;
+                for (int i = tid; i < n4; i += NT) {
+                    const float *sp = smem + pl * ppad + padL;
+                    const int a0 = row * LDR + x;
+                    const int a1 = (x + 2 >= w) ? (row + 1) * LDR + (x + 2 - w) : a0 + 2;
+                    float4 q;
+                    if (even_pad) {
+                        const float2 lo = *reinterpret_cast<const float2 *>(sp + a0);
+                        const float2 hi = *reinterpret_cast<const float2 *>(sp + a1);
+                        q = make_float4(lo.x, lo.y, hi.x, hi.y);
+                    } else {
+                        q = make_float4(sp[a0], sp[a0 + 1], sp[a1], sp[a1 + 1]);
+                    }
+                    store_nt(g4 + i, q);
+                    row += drow;
+                    x += dx;
+                    if (x >= w) { x -= w; ++row; }
+                    if (ppad) {
+                        pl += dpl;
+                        pe += dpe;
+                        if (pe >= hw) { pe -= hw; ++pl; }
+                    }
+                }
+            } else {
+                for (int i = tid; i < n4; i += NT) {
+                    float v[4];
+                    int r_ = row, x_ = x;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        v[c] = smem[r_ * LDR + padL + x_];
+                        if (++x_ == w) { x_ = 0; ++r_; }
+                    }
+                    store_nt(g4 + i, make_float4(v[0], v[1], v[2], v[3]));
+                    row += drow;
+                    x += dx;
+                    if (x >= w) { x -= w; ++row; }
+                }
             }
         }
         done = n4 << 2;
@@ -203,9 +244,9 @@ __device__ __forceinline__ void stage_raw(float *raw, const float *g, int nfloat
     }
 }
 
-// Zeroes the margins of nrows canvas rows and the all-zero row kept at index zrow.
+// Zeroes the margins of nrows canvas rows and the all-zero row kept at float offset zoff.
 template <int N, int NT = 256>
-__device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int w, int padL, int zrow,
+__device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int w, int padL, int zoff,
                                                     int tid)
 {
     constexpr int LDR = Canvas<N>::LDR;
@@ -214,7 +255,23 @@ __device__ __forceinline__ void zero_canvas_margins(float *smem, int nrows, int 
         for (int c = 0; c < padL; ++c) sp[c] = 0.0f;
         for (int c = padL + w; c < N; ++c) sp[c] = 0.0f;
     }
-    if (tid < N) smem[zrow * LDR + tid] = 0.0f;
+    if (tid < N) smem[zoff + tid] = 0.0f;
+}
+
+// Inverse transforms: floats to add between the canvases of two planes so that the plane stride, counted in
+// 16-byte slots, is `res` modulo `mod`.  The row pass writes canvas rows with 16-byte LDS accesses, 16 lanes per cycle; whether those 16
+// lanes (so many planes times so many rows, by the kernel's lane order) cover all 64 banks depends on that stride:
+//   * lanes that walk through 16 planes of one row (or 8 planes of two row pairs): an odd number of slots
+//     (mod 2, res 1), which h * LDR / 4 is by itself for odd h only;
+//   * one row per lane, TP planes fastest, then 16 / TP consecutive rows (a slot apart modulo 16 at N = 64 and 128,
+//     nine at N = 32): 16 / TP slots modulo 32 / TP.
+// 0 unless the copy runs in 16-byte pieces that cannot straddle two planes (even width, h * w a multiple of
+// four floats).
+inline int canvas_plane_pad(int ldr, int h, int w, int vec4, int mod, int res)
+{
+    if (!vec4 || (w & 1) != 0 || ((h * w) & 3) != 0) return 0;
+    const int q = (h * ldr / 4) % mod;
+    return 4 * ((res - q + mod) % mod);
 }
 
 // One launch can transform two tensors of the same FFT size (the two forward FFTs of a pass):
@@ -239,6 +296,7 @@ struct InvJob {
     int h, w, padU, padL;
     const float *bias;
     int bias_period, vec4;
+    int ppad;     // floats between the canvases of two planes beyond their rows (canvas_plane_pad)
     int tbl_off;
     Window win;
 };
