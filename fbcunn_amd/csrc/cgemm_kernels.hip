@@ -485,7 +485,8 @@ __global__ __launch_bounds__(256) void cgemm_ldsdirect_clock_kernel(const float2
 // is a quarter block (9 per SIMD for config 4).  Operands go straight from global memory into
 // the MFMA operand registers (each lane loads exactly the k' it feeds: 64 contiguous bytes of
 // a K-contiguous row, or one complex per row of a row-contiguous operand); LDS is used only
-// to add the partial accumulators.  Preconditions: M % 32 == N % 32 == 0, K % (16 * SK) == 0
+// to add the partial accumulators.  Preconditions: K % (16 * SK) == 0; M and N may be ragged (the lanes past
+// an edge load the last row or column again and store nothing)
 // (SK = waves that share one block: 4, 2 or 1; with SK = 1 a workgroup is four independent blocks).
 // ---------------------------------------------------------------------------------------
 template <int MODE>
@@ -559,6 +560,8 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
     const float2 *Bq = B + (long)q * N * K;
     float2 *Cq = C + (long)q * M * N;
 
+    // ragged M, N: the lanes past the edge load the last row / column again and store nothing
+    const int arow = (m0 + li < M) ? m0 + li : M - 1, bcol = (n0 + li < N) ? n0 + li : N - 1;
     const int kq = K / SK;                    // this wave's share of K (a multiple of 16)
     const int kbeg = ks * kq, nkt = kq >> 4;  // K-tiles of 16 complex
 
@@ -570,16 +573,16 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
         if constexpr (SK == 1) {
             // long K loop per wave: explicit register double buffering, loads pinned ahead of the MFMAs
             float a0[16], b0[16], a1[16], b1[16];
-            splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg, h, a0, b0);
+            splitk_load<MODE>(Aq, Bq, M, N, K, arow, bcol, kbeg, h, a0, b0);
             int kt = 0;
             for (; kt + 1 < nkt; kt += 2) {
-                splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * (kt + 1), h, a1, b1);
+                splitk_load<MODE>(Aq, Bq, M, N, K, arow, bcol, kbeg + 16 * (kt + 1), h, a1, b1);
                 __builtin_amdgcn_sched_barrier(0);
                 splitk_mfma<MODE>(a0, b0, p1, p2, p3);
                 __builtin_amdgcn_sched_barrier(0);
                 // the last prefetch of an even count re-reads the final tile and is not used
                 const int knext = (kt + 2 < nkt) ? kt + 2 : kt + 1;
-                splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * knext, h, a0, b0);
+                splitk_load<MODE>(Aq, Bq, M, N, K, arow, bcol, kbeg + 16 * knext, h, a0, b0);
                 __builtin_amdgcn_sched_barrier(0);
                 splitk_mfma<MODE>(a1, b1, p1, p2, p3);
                 __builtin_amdgcn_sched_barrier(0);
@@ -590,7 +593,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
             // previous tile's MFMAs, and at about 64 registers per lane five workgroups share a CU
             float a[16], b[16];
             for (int kt = 0; kt < nkt; ++kt) {
-                splitk_load<MODE>(Aq, Bq, M, N, K, m0 + li, n0 + li, kbeg + 16 * kt, h, a, b);
+                splitk_load<MODE>(Aq, Bq, M, N, K, arow, bcol, kbeg + 16 * kt, h, a, b);
                 splitk_mfma<MODE>(a, b, p1, p2, p3);
             }
         }
@@ -605,6 +608,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
         for (int r = 0; r < 16; ++r) {
             // accumulator register r of lane (li, h) is C[8*(r/4) + 4*h + r%4][li] of the block
             const int row = m0 + 8 * (r / 4) + 4 * h + (r % 4);
+            if (row >= M || n0 + li >= N) continue;
             float2 v = make_float2(alpha * cre[r], alpha * cim[r]);
             float2 *dst = Cq + (long)row * N + n0 + li;
             if (accumulate & RESULT_ACCUMULATE) {
@@ -635,6 +639,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
                 sim += red[w0 + v][16 + r][lane];
             }
             const int row = m0 + 8 * (r / 4) + 4 * h + (r % 4);
+            if (row >= M || n0 + li >= N) continue;
             float2 v = make_float2(alpha * sre, alpha * sim);
             float2 *dst = Cq + (long)row * N + n0 + li;
             if (accumulate & RESULT_ACCUMULATE) {
@@ -705,7 +710,7 @@ template <int MODE, int SK>
 static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_freq, int m, int n,
                                 int k, float alpha, int accumulate, FreqMap fm, hipStream_t s)
 {
-    const int tm = m / 32, tn = n / 32;
+    const int tm = (m + 31) / 32, tn = (n + 31) / 32;
     const long tot32 = (long)n_freq * tm * tn;
     const long wgs = (tot32 * SK + 3) / 4;
     const int chunk = (int)((wgs + 7) / 8);
@@ -733,8 +738,9 @@ static int splitk_override() { return g_force_variant.load(std::memory_order_rel
 //    256x96x64 conj(A)^T B takes 268 us (284 with 64x96 tiles by six waves, 321 with the register-fed
 //    kernel); 64x96x256 A B is as fast either way (251 us) and keeps the register-fed kernel;
 //  * at least 4 full 64x64 tiles per CU, or at least one and K >= 32, and 64-aligned M, N: LDS-direct tiles;
-//  * otherwise, if M, N are multiples of 32 and K of 16: the register-fed kernel, with more
-//    waves sharing one block's K range the fewer blocks there are per SIMD;
+//  * otherwise, if K is a multiple of 16 and M, N are multiples of 32 (or the problem is small, or a side is
+//    under 32): the register-fed kernel, with more waves sharing one block's K range the fewer blocks there
+//    are per SIMD;
 //  * anything else: register-staged LDS tiles with bounds checks.
 enum Variant { V_INVALID, V_HYBRID, V_TILES32, V_SPLIT4, V_SPLIT2, V_SPLIT1, V_TILES, V_STAGED };
 struct Choice {
@@ -750,7 +756,7 @@ static Choice choose_variant(int mode, const float *A, const float *B, int n_fre
     const bool aligned16 = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0;
     const int force = splitk_override();
     const bool direct_ok = (m % 64) == 0 && (n % 64) == 0 && (k % 16) == 0 && aligned16;
-    const long tot32 = (long)n_freq * (m / 32) * (n / 32);
+    const long tot32 = (long)n_freq * ((m + 31) / 32) * ((n + 31) / 32);
     if (direct_ok && (k % 64) == 0 &&
         (force == 9 || (force < 0 && total >= 256 && total < 8 * 256 && total % 256 <= 128))) {
         const int t64 = tilesM * tilesN;
@@ -765,8 +771,13 @@ static Choice choose_variant(int mode, const float *A, const float *B, int n_fre
     // 16.9 against 21.0 us, 512 tiles 17.3 against 21.6, 768 tiles 24.4 against 32.1, 256 tiles 11.1 against 11.9;
     // 130 x 128x128x32: 8.5 against 10.1)
     const bool prefer_direct = direct_ok && (force == 8 || (force < 0 && (total >= 4 * 256 || (total >= 256 && k >= 32))));
-    if (!prefer_direct && (m % 32) == 0 && (n % 32) == 0 && (k % 16) == 0 && aligned16 &&
-        tot32 * 4 < 0x7fffff00L) {
+    // Ragged M or N (the lanes past the edge are masked): the register-fed kernel for small problems and for
+    // sides under 32, where the staged kernel's 64 x 64 tiles are mostly empty (130 x 16x128x128: 9.6 against
+    // 17.9 us, 128x3x128: 9.4 against 18.0, 100x128x128: 27.2 against 28.0); from about four blocks per SIMD on
+    // the staged kernel's tiles win (528 x 100x64x64: 24.6 against 27.5 us, 2112 x 64x250x96: 239 against 276)
+    const bool ragged = (m % 32) != 0 || (n % 32) != 0;
+    const bool regs_ok = !ragged || force > 0 || tot32 < 4 * 1024 || m < 32 || n < 32;
+    if (!prefer_direct && regs_ok && (k % 16) == 0 && aligned16 && tot32 * 4 < 0x7fffff00L && force != 0) {
         int sk = 0;
         if (force >= 0) sk = (force == 8) ? 0 : force;
         else if (tot32 < 4 * 1024 && (k % 64) == 0) sk = 4;
@@ -875,14 +886,14 @@ __global__ __launch_bounds__(256) void cgemm_backward_kernel(MmJob j1, MmJob j2,
         const int wg = x * j1.chunk_split + j;
         if (wg >= j1.split_tiles) return;
         splitk_body<1, 4>(reinterpret_cast<float (*)[32][64]>(lds), j1.A, j1.B, j1.C, j1.M, j1.N, j1.K, j1.alpha,
-                          j1.accumulate, j1.M / 32, j1.N / 32, j1.split_tiles, wg, j1.q_direct, fm);
+                          j1.accumulate, (j1.M + 31) / 32, (j1.N + 31) / 32, j1.split_tiles, wg, j1.q_direct, fm);
         return;
     }
     j -= j1.chunk_split;
     const int wg = x * j2.chunk_split + j;
     if (wg >= j2.split_tiles) return;
     splitk_body<2, 4>(reinterpret_cast<float (*)[32][64]>(lds), j2.A, j2.B, j2.C, j2.M, j2.N, j2.K, j2.alpha,
-                      j2.accumulate, j2.M / 32, j2.N / 32, j2.split_tiles, wg, j2.q_direct, fm);
+                      j2.accumulate, (j2.M + 31) / 32, (j2.N + 31) / 32, j2.split_tiles, wg, j2.q_direct, fm);
 }
 
 // false: this problem's kernel is not one the grouped grid runs
@@ -903,7 +914,7 @@ static bool make_mm_job(int mode, const MmArgs &a, int n_freq, MmJob &j)
     j.q_direct = q_direct;
     j.direct_wgs = q_direct * (a.m / 64) * (a.n / 64);
     j.chunk_direct = (j.direct_wgs + 7) / 8;
-    j.split_tiles = (n_freq - q_direct) * (a.m / 32) * (a.n / 32);
+    j.split_tiles = (n_freq - q_direct) * ((a.m + 31) / 32) * ((a.n + 31) / 32);   // ragged sizes: split blocks only
     j.chunk_split = (j.split_tiles + 7) / 8;
     return true;
 }

@@ -32,6 +32,8 @@ SHAPES = [  # Q, m, n, k
     # a few rounds of 64x64 tiles with a ragged last one: whole rounds as LDS-direct tiles, the
     # left-over frequencies as split blocks, in one launch
     (70, 128, 128, 64), (300, 64, 64, 128), (33, 192, 128, 64),
+    # ragged M or N with K a multiple of 16: the register-fed kernel with its edge lanes masked
+    (130, 16, 128, 128), (7, 128, 3, 64), (9, 3, 5, 16), (40, 100, 120, 64), (5, 33, 31, 32), (3, 1, 1, 16), (11, 70, 130, 48),
     # one to four rounds of tiles whose last round is more than half full (or full): whole tiles throughout
     (60, 128, 256, 128), (130, 128, 128, 32), (64, 128, 128, 128),
     # N a multiple of 96 but not of 64 and at least 1024 64x96 blocks: 64x32 tiles by two waves
@@ -98,7 +100,9 @@ def test_against_oracle_contraction(nn, oracle, pass_):
 @pytest.mark.parametrize("shape,kernel", [((3, 128, 128, 128), "cgemm_splitk_kernel"), ((70, 128, 128, 64), "cgemm_hybrid_kernel"),
                                           ((300, 64, 64, 128), "cgemm_hybrid_kernel"), ((60, 128, 256, 128), "cgemm_ldsdirect_kernel"),
                                           ((130, 128, 128, 32), "cgemm_ldsdirect_kernel"), ((64, 128, 128, 128), "cgemm_ldsdirect_kernel"),
-                                          ((300, 128, 128, 64), "cgemm_ldsdirect_kernel"), ((6, 3, 5, 7), "cgemm_freq_kernel")])
+                                          ((300, 128, 128, 64), "cgemm_ldsdirect_kernel"), ((6, 3, 5, 7), "cgemm_freq_kernel"),
+                                          ((130, 16, 128, 128), "cgemm_splitk_kernel"), ((130, 128, 3, 128), "cgemm_splitk_kernel"),
+                                          ((2112, 64, 250, 96), "cgemm_freq_kernel")])
 def test_which_kernel_a_shape_takes(nn, shape, kernel):
     """The shape rule of the contraction: few tiles -> register-fed blocks with K shared by the waves; a few rounds
     of tiles with a thin last round -> tiles plus split blocks in one launch; otherwise whole tiles; ragged sizes ->
