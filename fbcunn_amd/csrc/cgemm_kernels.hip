@@ -537,7 +537,9 @@ __device__ __forceinline__ void splitk_mfma(const float (&a)[16], const float (&
 }
 
 // red: [wave][accumulator register][lane] partial sums (used when SK > 1)
-template <int MODE, int SK>
+// RAGGED: M, N need not be multiples of 32 (separate instantiations: the aligned code is the tail of the hybrid
+// and grouped kernels and stays as it was)
+template <int MODE, int SK, bool RAGGED = false>
 __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *__restrict__ A,
                                             const float2 *__restrict__ B, float2 *__restrict__ C, int M,
                                             int N, int K, float alpha, int accumulate, int tilesM,
@@ -561,7 +563,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
     float2 *Cq = C + (long)q * M * N;
 
     // ragged M, N: the lanes past the edge load the last row / column again and store nothing
-    const int arow = (m0 + li < M) ? m0 + li : M - 1, bcol = (n0 + li < N) ? n0 + li : N - 1;
+    const int arow = (!RAGGED || m0 + li < M) ? m0 + li : M - 1, bcol = (!RAGGED || n0 + li < N) ? n0 + li : N - 1;
     const int kq = K / SK;                    // this wave's share of K (a multiple of 16)
     const int kbeg = ks * kq, nkt = kq >> 4;  // K-tiles of 16 complex
 
@@ -608,7 +610,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
         for (int r = 0; r < 16; ++r) {
             // accumulator register r of lane (li, h) is C[8*(r/4) + 4*h + r%4][li] of the block
             const int row = m0 + 8 * (r / 4) + 4 * h + (r % 4);
-            if (row >= M || n0 + li >= N) continue;
+            if (RAGGED && (row >= M || n0 + li >= N)) continue;
             float2 v = make_float2(alpha * cre[r], alpha * cim[r]);
             float2 *dst = Cq + (long)row * N + n0 + li;
             if (accumulate & RESULT_ACCUMULATE) {
@@ -639,7 +641,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
                 sim += red[w0 + v][16 + r][lane];
             }
             const int row = m0 + 8 * (r / 4) + 4 * h + (r % 4);
-            if (row >= M || n0 + li >= N) continue;
+            if (RAGGED && (row >= M || n0 + li >= N)) continue;
             float2 v = make_float2(alpha * sre, alpha * sim);
             float2 *dst = Cq + (long)row * N + n0 + li;
             if (accumulate & RESULT_ACCUMULATE) {
@@ -652,7 +654,7 @@ __device__ __forceinline__ void splitk_body(float (*red)[32][64], const float2 *
     }
 }
 
-template <int MODE, int SK>
+template <int MODE, int SK, bool RAGGED>
 __global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restrict__ A,
                                                            const float2 *__restrict__ B,
                                                            float2 *__restrict__ C, int M, int N, int K,
@@ -663,7 +665,7 @@ __global__ __launch_bounds__(256) void cgemm_splitk_kernel(const float2 *__restr
     __shared__ float red[SK > 1 ? 4 : 1][32][64];
     const int wg = (int)(blockIdx.x % 8) * chunk + (int)(blockIdx.x / 8);
     if (wg >= total_wgs) return;
-    splitk_body<MODE, SK>(red, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, total_tiles, wg, 0, fm);
+    splitk_body<MODE, SK, RAGGED>(red, A, B, C, M, N, K, alpha, accumulate, tilesM, tilesN, total_tiles, wg, 0, fm);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -715,10 +717,14 @@ static hipError_t launch_splitk(const float *A, const float *B, float *C, int n_
     const long wgs = (tot32 * SK + 3) / 4;
     const int chunk = (int)((wgs + 7) / 8);
     note_kernel("cgemm_splitk_kernel", MODE, SK, (long)chunk * 8 * 256);
-    FBFC_LAUNCH((cgemm_splitk_kernel<MODE, SK>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s,
-                       reinterpret_cast<const float2 *>(A), reinterpret_cast<const float2 *>(B),
-                       reinterpret_cast<float2 *>(C), m, n, k, alpha, accumulate, tm, tn, (int)tot32,
-                       (int)wgs, chunk, fm);
+    const float2 *A2 = reinterpret_cast<const float2 *>(A), *B2 = reinterpret_cast<const float2 *>(B);
+    float2 *C2 = reinterpret_cast<float2 *>(C);
+    if ((m % 32) != 0 || (n % 32) != 0)
+        FBFC_LAUNCH((cgemm_splitk_kernel<MODE, SK, true>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s, A2, B2, C2,
+                    m, n, k, alpha, accumulate, tm, tn, (int)tot32, (int)wgs, chunk, fm);
+    else
+        FBFC_LAUNCH((cgemm_splitk_kernel<MODE, SK, false>), dim3((unsigned)(chunk * 8)), dim3(256), 0, s, A2, B2, C2,
+                    m, n, k, alpha, accumulate, tm, tn, (int)tot32, (int)wgs, chunk, fm);
     return hipGetLastError();
 }
 
@@ -886,14 +892,14 @@ __global__ __launch_bounds__(256) void cgemm_backward_kernel(MmJob j1, MmJob j2,
         const int wg = x * j1.chunk_split + j;
         if (wg >= j1.split_tiles) return;
         splitk_body<1, 4>(reinterpret_cast<float (*)[32][64]>(lds), j1.A, j1.B, j1.C, j1.M, j1.N, j1.K, j1.alpha,
-                          j1.accumulate, (j1.M + 31) / 32, (j1.N + 31) / 32, j1.split_tiles, wg, j1.q_direct, fm);
+                          j1.accumulate, j1.M / 32, j1.N / 32, j1.split_tiles, wg, j1.q_direct, fm);
         return;
     }
     j -= j1.chunk_split;
     const int wg = x * j2.chunk_split + j;
     if (wg >= j2.split_tiles) return;
     splitk_body<2, 4>(reinterpret_cast<float (*)[32][64]>(lds), j2.A, j2.B, j2.C, j2.M, j2.N, j2.K, j2.alpha,
-                      j2.accumulate, (j2.M + 31) / 32, (j2.N + 31) / 32, j2.split_tiles, wg, j2.q_direct, fm);
+                      j2.accumulate, j2.M / 32, j2.N / 32, j2.split_tiles, wg, j2.q_direct, fm);
 }
 
 // false: this problem's kernel is not one the grouped grid runs
@@ -903,7 +909,7 @@ static bool make_mm_job(int mode, const MmArgs &a, int n_freq, MmJob &j)
     int q_direct;
     if (ch.v == V_HYBRID) q_direct = ch.q_direct;
     else if (ch.v == V_TILES) q_direct = n_freq;
-    else if (ch.v == V_SPLIT4) q_direct = 0;
+    else if (ch.v == V_SPLIT4 && (a.m % 32) == 0 && (a.n % 32) == 0) q_direct = 0;
     else return false;
     j.A = reinterpret_cast<const float2 *>(a.A);
     j.B = reinterpret_cast<const float2 *>(a.B);
@@ -914,7 +920,7 @@ static bool make_mm_job(int mode, const MmArgs &a, int n_freq, MmJob &j)
     j.q_direct = q_direct;
     j.direct_wgs = q_direct * (a.m / 64) * (a.n / 64);
     j.chunk_direct = (j.direct_wgs + 7) / 8;
-    j.split_tiles = (n_freq - q_direct) * ((a.m + 31) / 32) * ((a.n + 31) / 32);   // ragged sizes: split blocks only
+    j.split_tiles = (n_freq - q_direct) * (a.m / 32) * (a.n / 32);
     j.chunk_split = (j.split_tiles + 7) / 8;
     return true;
 }
