@@ -81,21 +81,42 @@ __device__ __forceinline__ void copy_canvas(float *smem, float *g, int nrows, in
                         }
                     }
                 }
+                if ((w & 1) == 0) {
+                    // even width: each half of a piece lies in one canvas row
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int i = i0 + NT * u;
-                    if (i < n4) {
-                        const float v[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
-                        int r_ = row, x_ = x;
-#pragma unroll
-                        for (int c = 0; c < 4; ++c) {
-                            smem[r_ * LDR + padL + x_] = v[c];
-                            if (++x_ == w) { x_ = 0; ++r_; }
+                    for (int u = 0; u < U; ++u) {
+                        const int i = i0 + NT * u;
+                        if (i < n4) {
+                            float *a0 = smem + row * LDR + padL + x;
+                            float *a1 = (x + 2 >= w) ? smem + (row + 1) * LDR + padL + (x + 2 - w) : a0 + 2;
+                            if ((padL & 1) == 0) {
+                                *reinterpret_cast<float2 *>(a0) = make_float2(q[u].x, q[u].y);
+                                *reinterpret_cast<float2 *>(a1) = make_float2(q[u].z, q[u].w);
+                            } else {
+                                a0[0] = q[u].x; a0[1] = q[u].y; a1[0] = q[u].z; a1[1] = q[u].w;
+                            }
                         }
+                        row += drow;
+                        x += dx;
+                        if (x >= w) { x -= w; ++row; }
                     }
-                    row += drow;
-                    x += dx;
-                    if (x >= w) { x -= w; ++row; }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int i = i0 + NT * u;
+                        if (i < n4) {
+                            const float v[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+                            int r_ = row, x_ = x;
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) {
+                                smem[r_ * LDR + padL + x_] = v[c];
+                                if (++x_ == w) { x_ = 0; ++r_; }
+                            }
+                        }
+                        row += drow;
+                        x += dx;
+                        if (x >= w) { x -= w; ++row; }
+                    }
                 }
             }
         } else {
